@@ -82,8 +82,7 @@ __device__ __forceinline__ auto ld_raw8(const void* base, size_t off) {
 // decode loop keeps its block ids in a VGPR (lane j = the block of the wave's j-th chunk,
 // loaded once) and reads them with readlane: an SGPR, no memory instruction in the loop.
 // With a per-chunk bt[] load instead, the in-order vmcnt made every iteration wait for the
-// previous chunk's K/V AND then an L2 round trip before the next chunk's loads could issue
-// (the ISA showed `s_waitcnt vmcnt(2)` right after the three bt loads at the loop top).
+// previous chunk's K/V AND then an L2 round trip before the next chunk's loads could issue.
 template <bool NT = false, bool F8 = false>
 __device__ __forceinline__ void load_chunk_blk(ChunkT<F8>& c, const void* __restrict__ k_cache,
                                                const void* __restrict__ v_cache, int blk,

@@ -15,7 +15,7 @@
 // other buffer under this tile's 64 MFMAs per wave.  A no-math probe of exactly this operand
 // stream runs as fast as hipBLASLt's whole GEMM, and the phase pipeline below measured ~stream +
 // math; the stream-first loop is 5-14 % faster than it (0.70-0.88x hipBLASLt dense, 0.97-1.11x
-// with the SwiGLU epilogue, profiles/r6_pgemm_isa_diff.md).  The phase pipeline (SCHED 1):
+// with the SwiGLU epilogue).  The phase pipeline (SCHED 1):
 // NB = 2 (plain store; two raw s_barriers per K tile):
 //   phase | counted wait + barrier           | ds_reads issued            | DMA issued
 //   1     | W right + A bottom of tile t     | B right + A bottom (t)     | W right, A bottom (t+1)
@@ -278,7 +278,7 @@ __device__ __forceinline__ void pg_mainloop(bf16x8* lds, const __amdgpu_buffer_r
     // requested right after this tile's barrier and streams under this tile's MFMAs.  The
     // no-math stream of these tiles (one tile in flight, the same pattern) runs as fast as
     // hipBLASLt's whole GEMM, while the phase pipeline above measured stream + math
-    // (profiles/r6_pgemm_isa_diff.md, "no-math stream").  One wait, one barrier per K tile.
+    // (the "no-math stream" probe).  One wait, one barrier per K tile.
     issue(H0{}, 0);
     issue(H1{}, 0);
     issue(H2{}, 0);
@@ -430,11 +430,9 @@ __device__ __forceinline__ void pg_mainloop(bf16x8* lds, const __amdgpu_buffer_r
 }
 
 // ------------------------------------------------------------------------------------------
-// SCHED 3: the unit-pipelined 4-wave body (built from the ISA of the library kernel that wins
-// the prefill shapes, hipBLASLt's MT256x256x64_MI16x16x1 "SK3" kernel: 4 waves of 128 x 128,
-// one wave per SIMD, 256 accumulators, every LDS fragment read and every LDS-DMA piece issued
-// BETWEEN MFMAs, 3 vmcnt waits and ~2 barriers per 64-deep K tile; profiles/
-// r6_pgemm_isa_diff.md).  Against the phase pipeline above (same tile, same waves) it drops:
+// SCHED 3: the unit-pipelined 4-wave body (4 waves of 128 x 128, one wave per SIMD, 256
+// accumulators, every LDS fragment read and every LDS-DMA piece issued BETWEEN MFMAs, 3 vmcnt
+// waits and ~2 barriers per 64-deep K tile).  Against the phase pipeline above (same tile, same waves) it drops:
 //   * runtime-selected waits (pg_wait's if-chain: s_cbranch + SALU per wait),
 //   * bursts of 16-24 fragment reads before the MFMAs that consume them one by one,
 //   * the four-quadrant split of the accumulators (a quadrant's 16 MFMAs per phase).
@@ -871,12 +869,12 @@ long pgemm_sk_ws_floats(int M, int N, int splits) {
 // K-loop issue schedule: AKAP_PGEMM_SCHED = 1 (phase pipeline, half-tiles requested 1.0-1.25
 // tiles ahead), 2 (early issue, 1.25-1.75 tiles ahead), 3 (4-wave unit body), 4 (default,
 // stream-first: the whole next tile under this tile's math, 5-14 % faster than 1 on the dense
-// verdict shapes, profiles/r6_pgemm_isa_diff.md; pg_mainloop), read once per process.  The
+// verdict shapes; pg_mainloop), read once per process.  The
 // decode split-K form (launch_pgemm_sk) keeps 1 / 2.
 int pgemm_sched() {
   static int v = [] {
     const char* e = getenv("AKAP_PGEMM_SCHED");
-    const int x = e ? atoi(e) : 4;  // default: the stream-first body (r6_pgemm_isa_diff.md)
+    const int x = e ? atoi(e) : 4;  // default: the stream-first body
     return (x >= 1 && x <= 4) ? x : 4;
   }();
   return v;
