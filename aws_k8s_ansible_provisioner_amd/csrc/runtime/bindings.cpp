@@ -161,6 +161,16 @@ PYBIND11_MODULE(_runtime, m) {
              }
              return step_info(i);
            })
+      .def("schedule_forced",
+           [](Scheduler& s, const std::vector<std::pair<int64_t, std::vector<int32_t>>>& entries,
+              py::dict bufs) {
+             BatchBuffers b = batch_buffers(s, bufs);
+             std::vector<int32_t> rows;
+             StepInfo i = s.schedule_forced(entries, b, rows);
+             py::dict d = step_info(i);
+             d["entry_row"] = rows;
+             return d;
+           })
       .def("update",
            [](Scheduler& s, py::array_t<int64_t, py::array::c_style> toks) {
              std::vector<int64_t> ids;

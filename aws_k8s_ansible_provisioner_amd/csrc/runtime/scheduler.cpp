@@ -412,6 +412,16 @@ StepInfo Scheduler::schedule(BatchBuffers& buf) {
   prefill_only_run_ = (info.is_prefill && info.num_decode == 0 && any_decode)
                           ? prefill_only_run_ + 1 : 0;
 
+  flatten(sched, info, buf, sampled, true);
+  pending_.push_back(std::move(sampled));
+  last_pure_decode_ = !info.is_prefill && info.num_seqs > 0;
+  return info;
+}
+
+void Scheduler::flatten(const std::vector<std::pair<Request*, int>>& sched, StepInfo& info,
+                        BatchBuffers& buf, std::vector<int64_t>& sampled, bool do_sample) {
+  const int bs = cfg_.block_size;
+  const int mb = cfg_.max_blocks_per_seq;
   // ---------------- flatten ----------------
   int step_rows = cfg_.tile_rows;
   if (cfg_.tile_rows_short > 0 && info.is_prefill) {
@@ -455,7 +465,7 @@ StepInfo Scheduler::schedule(BatchBuffers& buf) {
       }
     }
     r->num_computed = kv;
-    const bool sample = kv == (int)r->tokens.size();
+    const bool sample = do_sample && kv == (int)r->tokens.size();
     buf.sample_mask[s] = sample ? 1 : 0;
     if (sample) {
       buf.temperature[ns] = r->temperature;
@@ -474,8 +484,80 @@ StepInfo Scheduler::schedule(BatchBuffers& buf) {
   info.num_tokens = T;
   info.num_tiles = tiles;
   info.num_samples = ns;
-  pending_.push_back(std::move(sampled));
-  last_pure_decode_ = !info.is_prefill && info.num_seqs > 0;
+}
+
+
+StepInfo Scheduler::schedule_forced(
+    const std::vector<std::pair<int64_t, std::vector<int32_t>>>& entries, BatchBuffers& buf,
+    std::vector<int32_t>& entry_row) {
+  StepInfo info;
+  pending_.clear();  // replayed steps sample nothing: no update() is due for them
+  last_pure_decode_ = false;
+  if ((int)entries.size() > cfg_.max_num_seqs)
+    throw std::invalid_argument("schedule_forced: more entries than max_num_seqs");
+  // validate everything before touching any state: a refused step changes nothing
+  int total = 0;
+  for (size_t e = 0; e < entries.size(); ++e) {
+    const auto& en = entries[e];
+    if (en.second.empty()) throw std::invalid_argument("schedule_forced: entry without tokens");
+    for (size_t o = 0; o < e; ++o)
+      if (entries[o].first == en.first)
+        throw std::invalid_argument("schedule_forced: a request appears twice in one step");
+    auto it = reqs_.find(en.first);
+    int have = 0;
+    if (it != reqs_.end()) {
+      const Request& r = *it->second;
+      if (r.status != RUNNING || r.num_computed != (int)r.tokens.size())
+        throw std::invalid_argument("schedule_forced: request is not a live replayed one");
+      have = (int)r.tokens.size();
+    } else if ((int)running_.size() + 1 > cfg_.max_num_seqs) {
+      throw std::invalid_argument("schedule_forced: no free sequence slot");
+    }
+    if (have + (int)en.second.size() > cfg_.max_model_len)
+      throw std::invalid_argument("schedule_forced: request longer than max_model_len");
+    total += (int)en.second.size();
+  }
+  if (total > buf.cap_tokens) throw std::invalid_argument("schedule_forced: step too large");
+  // single-token rows lead the batch (the decode rows of a mixed step), chunks follow; both
+  // keep the caller's order
+  std::vector<int> order;
+  bool any_chunk = false;
+  for (size_t e = 0; e < entries.size(); ++e)
+    if (entries[e].second.size() == 1) order.push_back((int)e);
+  const int singles = (int)order.size();
+  for (size_t e = 0; e < entries.size(); ++e)
+    if (entries[e].second.size() != 1) { order.push_back((int)e); any_chunk = true; }
+  std::vector<std::pair<Request*, int>> sched;
+  for (int e : order) {
+    const auto& en = entries[e];
+    auto it = reqs_.find(en.first);
+    Request* r;
+    if (it == reqs_.end()) {
+      auto nr = std::make_unique<Request>();
+      nr->id = en.first;
+      nr->ignore_eos = true;
+      nr->max_tokens = cfg_.max_model_len;
+      nr->prefix_checked = true;  // every token of a replayed request is computed here
+      nr->status = RUNNING;
+      r = nr.get();
+      running_.push_back(r);
+      reqs_.emplace(en.first, std::move(nr));
+    } else {
+      r = it->second.get();
+    }
+    r->tokens.insert(r->tokens.end(), en.second.begin(), en.second.end());
+    r->num_prompt = (int)r->tokens.size();
+    if (!ensure_blocks(*r, (int)r->tokens.size()))
+      throw std::runtime_error("schedule_forced: out of KV blocks");
+    sched.emplace_back(r, (int)en.second.size());
+  }
+  info.num_decode = any_chunk ? singles : (int)sched.size();
+  info.is_prefill = any_chunk ? 1 : 0;
+  std::vector<int64_t> sampled;
+  // a pure single-token step runs the decode path, sampler included (its picks are dropped)
+  flatten(sched, info, buf, sampled, !any_chunk);
+  entry_row.assign(entries.size(), 0);
+  for (size_t s = 0; s < order.size(); ++s) entry_row[order[s]] = buf.q_start[s];
   return info;
 }
 

@@ -136,6 +136,17 @@ class Scheduler {
   // requests that a free sequence slot could admit, a running sequence outside the in-flight
   // batch, no KV blocks, nothing left).
   StepInfo schedule_lookahead(BatchBuffers& buf, int64_t* src_rows);
+  // Replay: the caller dictates the step.  Each entry (id, tokens) appends `tokens` to request
+  // `id` (admitted as a running request at its first entry; no prefix-cache lookup, nothing is
+  // sampled from it) and schedules exactly those tokens on top of what earlier steps left in
+  // the request's blocks.  Rows are laid out as in a mixed step: single-token entries lead
+  // (num_decode of them beside chunks; a step of single tokens only is a pure decode step),
+  // chunks follow; entry_row[e] is the flattened row of entry e's first token.  No update()
+  // follows such a step; a request ends by abort_request() + release().  Throws, leaving the
+  // state untouched, when the step does not fit (sequence slots, token buffer, model length);
+  // runs out of KV blocks -> std::runtime_error.
+  StepInfo schedule_forced(const std::vector<std::pair<int64_t, std::vector<int32_t>>>& entries,
+                           BatchBuffers& buf, std::vector<int32_t>& entry_row);
   // tokens[i] is the sample for the i-th sampled sequence of the last step.
   // Emits (id, token, finish_reason, is_first) events only for sequences that got their
   // first token, finished, or stream -- O(events) host work per step, not O(batch).
@@ -201,6 +212,10 @@ class Scheduler {
   void schedule_decodes(std::vector<std::pair<Request*, int>>& sched, StepInfo& info,
                         int& budget);
   void schedule_prefills(std::vector<std::pair<Request*, int>>& sched, int& budget);
+  // writes the chosen (request, q_len) rows into the batch buffers and advances num_computed;
+  // do_sample: rows whose every token is then computed get a sampler row
+  void flatten(const std::vector<std::pair<Request*, int>>& sched, StepInfo& info,
+               BatchBuffers& buf, std::vector<int64_t>& sampled, bool do_sample);
   void publish_full_blocks(Request& r);
   void preempt(Request& r);
   void finish(Request& r, int reason);

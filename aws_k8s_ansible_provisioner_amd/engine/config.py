@@ -40,11 +40,15 @@ class EngineConfig:
     # samples) before waiting for step N, so host bookkeeping and the graph launch overlap
     # the GPU (single-rank engines with hipGraphs; AKAP_ASYNC_DECODE=0 disables)
     async_decode: bool = True
+    dtype: str = "bfloat16"                   # "bfloat16" | "float32" (models that have fp32 kernels)
+    logits_only: bool = False                 # steps return logits, nothing is sampled (replay)
 
     def __post_init__(self) -> None:
         # the K cache stores each 32-token chunk in MFMA-fragment order (ops/reference.py)
         if self.block_size <= 0 or self.block_size % 32:
             raise ValueError(f"block_size must be a multiple of 32, got {self.block_size}")
+        if self.dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"dtype must be bfloat16 or float32, got {self.dtype}")
         if self.kv_cache_dtype not in ("auto", "bf16", "bfloat16", "fp8", "fp8_e4m3"):
             raise ValueError(f"kv_cache_dtype must be auto or fp8, got {self.kv_cache_dtype}")
 

@@ -556,6 +556,40 @@ class LLMEngine:
             probe = getattr(self, "kv_ipc_state", None)  # set by the serving layer (decode)
             m.kv_ipc.set(1.0 if probe is not None and probe() else 0.0, model_name=name)
 
+    # ------------------------------------------------------------------ replay
+    def replay_step(self, entries: list, end: Iterable = ()) -> np.ndarray:
+        """Teacher-forced step: entries = [(request name, new token ids, wanted places)].
+        Every entry's tokens are appended to its request (admitted at its first entry) and run
+        as ONE batch on top of the KV its earlier steps left -- single tokens beside chunks,
+        through the scheduler's block tables and the runner's mixed / decode paths.  Returns
+        fp32 logits [sum of wanted places, vocab], in the order of the entries and of their
+        wanted places (indices into the entry's tokens).  Requests named in `end` give their
+        blocks back after the step.  Nothing is sampled; such requests never enter step()."""
+        with self._lock:
+            forced = []
+            for name, toks, _ in entries:
+                iid = self.by_name.get(name)
+                if iid is None:
+                    iid = next(self._ids)
+                    self.by_name[name] = iid
+                forced.append((iid, [int(t) for t in toks]))
+            info = self.sched.schedule_forced(forced, self.runner.host_buffers())
+            rows = []
+            for (name, toks, want), r0 in zip(entries, info["entry_row"]):
+                for w in want:
+                    if not 0 <= int(w) < len(toks):
+                        raise ValueError(f"wanted place {w} outside the {len(toks)} tokens of "
+                                         f"{name!r}")
+                    rows.append(r0 + int(w))
+            logits = self.runner.step_logits(info, rows)
+            for name in end:
+                iid = self.by_name.pop(name, None)
+                if iid is not None:
+                    self.sched.abort_request(iid)
+                    self.sched.release(iid)
+        self.steps += 1
+        return logits.numpy()
+
     # ------------------------------------------------------------------ offline API
     def generate(self, prompts: Iterable, params: Optional[SamplingParams] = None,
                  prompt_ids: Optional[list] = None) -> list[RequestOutput]:

@@ -22,8 +22,9 @@ import torch
 from ..utils import profiling
 from .. import ops
 from ..models import moe as moe_mod
+from ..models import model_class
 from ..models.config import ModelConfig
-from ..models.transformer import AttnBatch, DecoderLM
+from ..models.transformer import AttnBatch
 from ..parallel.state import ParallelState, drain_pending_collectives, get_state
 from .config import EngineConfig
 
@@ -43,6 +44,10 @@ DECODE_FIELDS = ("input_ids", "positions", "slots", "seeds", "seq_lens", "temper
 # its peers' custom collectives time out inside a replayed graph
 _FAULT_SKIP_REPLAY = int(os.environ.get("AKAP_FAULT_SKIP_REPLAY", "0"))
 
+def tile_plan_of(model):
+    return getattr(model, "prefill_tile_plan", None)
+
+
 class ModelRunner:
     def __init__(self, ecfg: EngineConfig, mcfg: ModelConfig,
                  pstate: Optional[ParallelState] = None, log=print):
@@ -50,16 +55,25 @@ class ModelRunner:
         self.ps = pstate or get_state()
         self.log = log
         dev = ecfg.resolved_device()
+        cls = model_class(mcfg)
+        # models on the stream kernels (ops.stream) need the core library only for the sampler
+        # and the staging kernel: a step that returns logits alone runs without it
+        self._core_native = dev == "cuda" and (getattr(cls, "gemm_tunable", True)
+                                               or not ecfg.logits_only)
         if dev == "cuda":
             self.device = torch.device("cuda", torch.cuda.current_device())
-            ops.load_native(required=True)  # GPU path never falls back to eager PyTorch
+            if self._core_native:
+                ops.load_native(required=True)  # GPU path never falls back to eager PyTorch
         else:
             self.device = torch.device("cpu")
         self.is_gpu = self.device.type == "cuda"
         t0 = time.time()
-        self.model = DecoderLM(mcfg, self.device, seed=ecfg.seed, pstate=self.ps,
-                               max_model_len=ecfg.max_model_len, init_std=ecfg.init_std,
-                               full_then_shard=ecfg.shard_init == "full")
+        dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[ecfg.dtype]
+        if dev == "cuda" and dtype not in getattr(cls, "dtypes", (torch.bfloat16,)):
+            raise ValueError(f"{mcfg.name}: the GPU kernels of this model run in bfloat16 only")
+        self.model = cls(mcfg, self.device, dtype=dtype, seed=ecfg.seed, pstate=self.ps,
+                         max_model_len=ecfg.max_model_len, init_std=ecfg.init_std,
+                         full_then_shard=ecfg.shard_init == "full")
         if ecfg.load_format == "safetensors" and ecfg.weights_path:
             from .weights import load_safetensors_dir
 
@@ -69,6 +83,8 @@ class ModelRunner:
         self.bs = ecfg.block_size
         self.max_blocks = math.ceil(ecfg.max_model_len / self.bs)
         self.G = self.model.hq // self.model.hkv
+        # models with their own prefill attention kernels give the tile map's granularity
+        tile_plan = getattr(self.model, "prefill_tile_plan", None)
         self.max_seqs = ecfg.max_num_seqs
         # a mixed step holds a full prefill token budget plus one decode row per sequence
         self.cap_tokens = ecfg.max_num_batched_tokens + self.max_seqs
@@ -87,6 +103,8 @@ class ModelRunner:
             self.tile_rows_short = 0
             if self.tile_rows == 256 and ecfg.kv_cache_dtype.startswith("fp8"):
                 self.tile_rows = 128  # the 256-row kernel needs a bf16 KV cache
+        if tile_plan is not None:
+            self.G, self.tile_rows, self.tile_rows_short = tile_plan()
         self.cap_tiles = self.cap_tokens * self.G // 64 + self.max_seqs + 1
         self.num_blocks = ecfg.num_gpu_blocks or self._derive_num_blocks()
         if self.ps.tp_size > 1:  # every TP rank must address the same block pool
@@ -125,6 +143,9 @@ class ModelRunner:
         # top-N alternatives of the last step's sampled rows: (token ids [n, N], log-probs)
         self.last_top: Optional[tuple] = None
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
+        # logits of the last eager decode step per batch size, and of each captured graph
+        self._step_logits: dict = {}
+        self._graph_logits: dict = {}
         # decode graphs whose sampler also runs the top-k / top-p threshold passes: captured on
         # first use by a batch that needs them (single-rank engines; multi-rank engines capture
         # their only graphs with the passes, since a lazy capture would issue collectives alone)
@@ -143,7 +164,8 @@ class ModelRunner:
         cache, fused decode attention.  AKAP_V_TAIL=0 restores the per-token cache write."""
         from ..models import transformer as tfm
 
-        return (self.is_gpu and self.kv_dtype == torch.bfloat16 and tfm.FUSED_DECODE and
+        return (self.is_gpu and getattr(self.model, "supports_v_tail", True) and
+                self.kv_dtype == torch.bfloat16 and tfm.FUSED_DECODE and
                 os.environ.get("AKAP_V_TAIL", "1") != "0" and
                 not (self.ecfg.kv_role == "decode" and self.ps.tp_size > 1))
 
@@ -177,7 +199,10 @@ class ModelRunner:
     # ------------------------------------------------------------------ sizing
     def _derive_num_blocks(self) -> int:
         elem = 1 if self.ecfg.kv_cache_dtype.startswith("fp8") else 2
-        per_block = self.mcfg.num_layers * 2 * self.model.hkv * self.bs * self.model.D * elem
+        if hasattr(self.model, "kv_block_bytes"):  # layers of unequal KV width
+            per_block = self.model.kv_block_bytes(self.bs, self.ecfg.kv_cache_dtype)
+        else:
+            per_block = self.mcfg.num_layers * 2 * self.model.hkv * self.bs * self.model.D * elem
         if not self.is_gpu:
             return max(64, min(4096, (self.max_seqs * self.ecfg.max_model_len) // self.bs + 8))
         torch.cuda.synchronize()
@@ -243,7 +268,7 @@ class ModelRunner:
         # the staging kernel needs the pinned buffers' device mapping: probe it once, fall back
         # to hipMemcpyAsync where the host allocator does not provide one
         self._h2d_kernel = False
-        if self.is_gpu and H2D_KERNEL:
+        if self.is_gpu and H2D_KERNEL and self._core_native:
             try:
                 torch.ops.akap.h2d_stage(self.ddec[:16], self.hdecs[0][:16])
                 self._h2d_kernel = True
@@ -262,8 +287,10 @@ class ModelRunner:
         self._follower_slot = 0
         self._replays = 0
         self.out_logprobs = torch.zeros(S, dtype=torch.float32, device=self.device)
+        # split-KV scratch of the D = 128 decode kernel (models on other kernels keep their own)
         self.workspace = ops.decode_workspace(S, self.model.hkv, self.G, self.num_parts,
-                                              self.device)
+                                              self.device) if tile_plan_of(self.model) is None \
+            else None
 
     def host_buffers(self) -> dict:
         return self.np
@@ -398,9 +425,10 @@ class ModelRunner:
         return {k: self._dpre[o:o + n * self.h[k].element_size()].view(self.h[k].dtype)
                 for k, (o, n) in lay.items()}
 
-    def execute_prefill(self, info: dict) -> torch.Tensor:
-        """A step with prefill chunks; under mixed batching its leading `num_decode` rows are
-        running sequences' decode tokens (eager, same forward)."""
+    def _forward_prefill(self, info: dict):
+        """Stage a step with prefill chunks and run the model on it; under mixed batching its
+        leading `num_decode` rows are running sequences' decode tokens (eager, same forward).
+        Returns the final hidden rows [T, d] and the staged device views."""
         T, B, nt, ns = info["num_tokens"], info["num_seqs"], info["num_tiles"], info["num_samples"]
         mb = self.max_blocks
         v = self._stage_prefill(info)
@@ -430,6 +458,14 @@ class ModelRunner:
             from ..parallel import comm
 
             comm.check_deferred()
+        return h, v
+
+    def execute_prefill(self, info: dict) -> torch.Tensor:
+        """A step with prefill chunks: forward, then the sampler on the rows that finish their
+        prompt."""
+        ns = info["num_samples"]
+        h, v = self._forward_prefill(info)
+        lidx = v["logits_idx"]
         if ns == 0:
             # a chunk that samples nothing (a long prompt's inner chunk): the caller's
             # device->host copy of zero tokens does not wait for the GPU, but the H2D copies
@@ -444,6 +480,39 @@ class ModelRunner:
             logits = logits.float()  # the GPU sampler reads bf16 logits directly
         toks, _ = self._sample(logits, ns, info.get("extras"), src=v)
         return toks
+
+    def step_logits(self, info: dict, rows) -> torch.Tensor:
+        """Run a scheduled step and return fp32 logits [len(rows), vocab] of the flattened
+        token rows `rows` instead of sampled tokens (trace replay, scoring).  A step with
+        chunks runs the eager mixed path; a step of single tokens only runs the decode path
+        of generation: the hipGraph of its batch-size bucket when captured."""
+        if info["is_prefill"]:
+            h, _ = self._forward_prefill(info)
+            if not len(rows):
+                if self.is_gpu:  # the staged H2D copies must finish before the buffers change
+                    torch.cuda.current_stream().synchronize()
+                return torch.empty(0, self.mcfg.vocab_size)
+            idx = torch.as_tensor(list(rows), dtype=torch.int64).to(self.device)
+            return self.model.compute_logits(h.index_select(0, idx)).float().cpu()
+        B = info["num_seqs"]
+        n = self._bucket(B) if self.graphs else B
+        self._pad_host(B, n)
+        self._stage_decode(n)
+        graph = self.graphs.get(n) if self.graphs else None
+        if graph is not None:
+            mode = "plain" if self.ecfg.logits_only else (
+                "filtered" if self._peer_step else self._sample_mode(B))
+            (graph if (mode, n) not in self.graphs_v else self.graphs_v[(mode, n)]).replay()
+            logits = self._graph_logits[(mode, n)]
+        else:
+            self._decode_body(n)
+            logits = self._step_logits[n]
+        if not len(rows):
+            if self.is_gpu:
+                torch.cuda.current_stream().synchronize()
+            return torch.empty(0, self.mcfg.vocab_size)
+        idx = torch.as_tensor(list(rows), dtype=torch.int64).to(self.device)
+        return logits.index_select(0, idx).float().cpu()
 
     def decode_partitions(self, n: int) -> tuple[int, int]:
         """Split-KV plan for a decode batch of n sequences.  Enough (seq, kv-head)
@@ -486,7 +555,12 @@ class ModelRunner:
         h = self.model.forward(dd["input_ids"][:n], batch, self.k_caches, self.v_caches)
         # sampler reads bf16 logits directly (no [n, V] fp32 cast pass)
         logits = self.model.compute_logits(h)
-        self._sample(logits, n, extras, src=dd)
+        # kept for step_logits(): under capture this is the graph's own output buffer, alive
+        # (and not reused by later captures in the shared pool) while referenced here
+        self._step_logits[n] = logits
+        if not self.ecfg.logits_only:
+            self._sample(logits if logits.dtype == torch.bfloat16 or not self.is_gpu
+                         else logits.to(torch.bfloat16), n, extras, src=dd)
         if self._ep_moe:
             moe_mod.ep_overflow_reduce(self.device)
 
@@ -720,7 +794,8 @@ class ModelRunner:
                 "AKAP_TUNABLEOP_FILE", os.path.join(os.getcwd(), "tunableop_results.csv")))
         # safe static contents: every row is padding
         self._pad_host(0, self.max_seqs)
-        if os.environ.get("AKAP_GEMM_TUNE", "1") != "0":
+        if os.environ.get("AKAP_GEMM_TUNE", "1") != "0" and \
+                getattr(self.model, "gemm_tunable", True):
             # MoE models: the attention projections are tuned (the experts run the grouped
             # GEMM; tune_fused skips MoE layers)
             # per-(M, N, K) hipBLASLt vs MFMA-kernel choice on the real, cold layer weights
@@ -771,6 +846,8 @@ class ModelRunner:
         # "filtered", all captured here -- a capture while serving would race the P/D KV
         # receiver's work; multi-rank engines: "filtered" only, correct for every batch)
         modes = ["filtered"] if self._peer_step else ["plain", "greedy", "filtered"]
+        if self.ecfg.logits_only:
+            modes = ["plain"]  # nothing is sampled: one graph per bucket
         for mode in modes:
             self._capture_mode = mode
             for b in reversed(self.buckets):
@@ -782,6 +859,7 @@ class ModelRunner:
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g, pool=self.graph_pool, stream=stream):
                     self._decode_body(b)
+                self._graph_logits[(mode, b)] = self._step_logits[b]
                 if mode == modes[0]:
                     self.graphs[b] = g
                 else:

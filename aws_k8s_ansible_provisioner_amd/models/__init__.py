@@ -1,1 +1,12 @@
 from .config import ModelConfig, get_config, list_models  # noqa: F401
+
+
+def model_class(cfg: ModelConfig):
+    """The model implementation that serves `cfg` (by its arch)."""
+    if cfg.arch == "bidetar":
+        from .bidetar import BidetarLM
+
+        return BidetarLM
+    from .transformer import DecoderLM
+
+    return DecoderLM

@@ -18,7 +18,7 @@ from typing import Optional
 class ModelConfig:
     name: str
     hf_id: str
-    arch: str  # "qwen3" | "llama" | "mixtral" | "qwen3_moe"
+    arch: str  # "qwen3" | "llama" | "mixtral" | "qwen3_moe" | "bidetar" (LayeredConfig)
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -94,6 +94,136 @@ class ModelConfig:
                     else d["eos_token_id"][0]),
         )
 
+
+@dataclasses.dataclass
+class RotarySpec:
+    """Rotary positions on the first `dims` dimensions of every head (pairs (2i, 2i+1)):
+    f_i = base^(-2i/dims), optionally rescaled by wavelength (`scaling`: factor, low, high,
+    original -- the Llama-3.1 rule)."""
+    dims: int
+    base: float
+    scaling: Optional[dict] = None
+
+
+@dataclasses.dataclass
+class AttentionSpec:
+    """One attention mixer of a layered model: H query heads over G key/value heads of size
+    `dim`; chunk > 0 restricts a query to the keys of its own chunk of that many positions
+    (window > 0: to the last `window` keys); sink: a learned per-head logit in the softmax
+    denominator; gate: a per-head sigmoid gate on the head outputs; shared_kv: the values are
+    the key projection itself (before its norm and rotation)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rot: Optional[RotarySpec] = None
+    chunk: int = 0
+    window: int = 0
+    sink: bool = True
+    gate: bool = True
+    shared_kv: bool = True
+
+
+@dataclasses.dataclass
+class MlpSpec:
+    kind: str   # "dense": down(act(up h))
+    ff: int
+    act: str = "relu2"
+
+
+@dataclasses.dataclass
+class LayerSpec:
+    type: str                       # which mixer: "attention"
+    mixer: AttentionSpec
+    mlp: Optional[MlpSpec] = None   # None: the layer has no feed-forward
+
+
+@dataclasses.dataclass
+class LayeredConfig(ModelConfig):
+    """A model given as an explicit list of layers (each with its own mixer and feed-forward
+    sizes) over an fp32 residual stream, with an optional loop that runs a span of layers
+    several times with the same weights (each pass has its own KV cache).  The ModelConfig
+    fields hold the stack's maxima (heads, head size, ffn) for buffer sizing; num_layers is
+    the number of layer RUNS (= KV cache layers)."""
+    layer_specs: list = dataclasses.field(default_factory=list)
+    loop: Optional[tuple] = None    # (start, stop, times)
+    embed_scale: float = 1.0
+    residual_mult: float = 1.0
+
+    def layer_runs(self) -> list:
+        """Indices into layer_specs in execution order."""
+        n = len(self.layer_specs)
+        if not self.loop:
+            return list(range(n))
+        a, b, t = self.loop
+        return list(range(a)) + list(range(a, b)) * t + list(range(b, n))
+
+    def kv_bytes_per_token(self, tp: int = 1) -> int:
+        es = 4 if self.dtype == "float32" else 2
+        return sum(2 * self.layer_specs[i].mixer.kv_heads * self.layer_specs[i].mixer.dim * es
+                   for i in self.layer_runs())
+
+    def num_params(self) -> int:
+        d = self.hidden_size
+        n = 2 * self.vocab_size * d + d
+        for ls in self.layer_specs:
+            m = ls.mixer
+            n += d + (m.heads + m.kv_heads) * m.dim * (d + 2) + m.heads * (d + 1) \
+                + d * (m.heads * m.vdim + 1)
+            if ls.mlp is not None:
+                n += 2 * d * ls.mlp.ff
+        return n
+
+
+def bidetar_config(name: str, d: dict, max_position: int = 1 << 20) -> LayeredConfig:
+    """A Bidetar config.json: parallel layers (one norm feeds the attention mixer and the
+    feed-forward) of chunked sink attention with shared key/value projections."""
+    specs = []
+    for ly in d["layers"]:
+        if ly["type"] != "attention":
+            raise ValueError(f"Bidetar: unknown mixer type {ly['type']!r}")
+        m = ly["mixer"]
+        rot = m.get("rot")
+        rs = None
+        if rot:
+            rs = RotarySpec(int(rot["dims"]), float(rot["base"]), rot.get("scaling") or None)
+        mask = m.get("mask") or {}
+        if int(m.get("vdim", m["dim"])) != int(m["dim"]):
+            raise ValueError("Bidetar: the values are the key projection, vdim must equal dim")
+        mixer = AttentionSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                              dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                              scale=float(m["scale"]), rot=rs, chunk=int(mask.get("size") or 0))
+        if mixer.heads % mixer.kv_heads:
+            raise ValueError("Bidetar: heads must be a multiple of kv_heads")
+        ml = ly.get("mlp")
+        mlp = None
+        if ml is not None:
+            if ml.get("kind", "dense") != "dense":
+                raise ValueError(f"Bidetar: unknown feed-forward kind {ml.get('kind')!r}")
+            mlp = MlpSpec("dense", int(ml["ff"]))
+        specs.append(LayerSpec("attention", mixer, mlp))
+    lp = d.get("loop")
+    loop = None
+    if lp and int(lp.get("times", 1)) != 1 and int(lp["stop"]) > int(lp["start"]):
+        loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"]))
+        if not (0 <= loop[0] < loop[1] <= len(specs)) or loop[2] < 1:
+            raise ValueError(f"Bidetar: bad loop {lp}")
+    cfg = LayeredConfig(
+        name=name, hf_id=name, arch="bidetar", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]),
+        intermediate_size=max([ls.mlp.ff for ls in specs if ls.mlp is not None] or [0]),
+        num_layers=0, num_heads=max(ls.mixer.heads for ls in specs),
+        num_kv_heads=max(ls.mixer.kv_heads for ls in specs),
+        head_dim=max(ls.mixer.dim for ls in specs), rms_eps=float(d["norm"]["eps"]),
+        max_position=max_position, bos_id=0, eos_id=-1, layer_specs=specs, loop=loop,
+        embed_scale=float(d["embedding"]["scale"]), residual_mult=float(d["residual_mult"]))
+    cfg.num_layers = len(cfg.layer_runs())
+    return cfg
+
+
+# config.json readers of designs that do not use the HF key set, by their "architecture" value
+_NATIVE_READERS = {"Bidetar": bidetar_config}
 
 _REGISTRY: dict[str, ModelConfig] = {}
 
@@ -190,7 +320,11 @@ def get_config(name: str) -> ModelConfig:
     """Resolve a registry name, HF id, or a directory holding a HF config.json."""
     if os.path.isdir(name) and os.path.exists(os.path.join(name, "config.json")):
         with open(os.path.join(name, "config.json")) as f:
-            return ModelConfig.from_hf_dict(name, json.load(f))
+            d = json.load(f)
+        reader = _NATIVE_READERS.get(d.get("architecture"))
+        if reader is not None:
+            return reader(name, d)
+        return ModelConfig.from_hf_dict(name, d)
     key = name.lower()
     if key in _REGISTRY:
         return _REGISTRY[key]
