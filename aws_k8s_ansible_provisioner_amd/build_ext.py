@@ -28,7 +28,11 @@ import sysconfig
 PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 BUILD = os.path.join(PKG, "csrc", "build")
+STREAM_SRC = os.path.join(PKG, "csrc", "stream")
 ARCH = os.environ.get("AKAP_ARCH", "gfx950")
+# device code is compiled without packed-fp32 instructions (v_pk_*_f32): hipcc -O3 forms them
+# from ordinary float code, and some of their forms have given wrong results on this hardware
+NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
@@ -125,8 +129,8 @@ def build_kernels(force: bool = False, jobs: int = 8, log=None) -> str:
     for src in sorted(glob.glob(os.path.join(CSRC, "kernels", "*.hip"))):
         obj = os.path.join(BUILD, os.path.basename(src) + ".o")
         objs.append(obj)
-        cmd = [HIPCC, f"--offload-arch={ARCH}", *common, "-munsafe-fp-atomics", "-c", src, "-o",
-               obj]
+        cmd = [HIPCC, f"--offload-arch={ARCH}", *common, *NO_PACKED_FP32, "-munsafe-fp-atomics",
+               "-c", src, "-o", obj]
         digest = _digest([src] + headers, " ".join(cmd[:-3]))
         why = "forced" if force else _stale(obj, digest)
         if why:
@@ -166,6 +170,89 @@ def build_kernels(force: bool = False, jobs: int = 8, log=None) -> str:
             f.write(_digest(objs + [info_obj]) + "\n")
     else:
         log(f"reuse _C.so: built from this tree ({tree[:16]}, torch {tv})")
+    return out
+
+
+def stream_sources() -> list[str]:
+    return sorted(glob.glob(os.path.join(STREAM_SRC, "*.hip")) +
+                  glob.glob(os.path.join(STREAM_SRC, "*.h")) +
+                  glob.glob(os.path.join(STREAM_SRC, "*.cpp")) +
+                  [os.path.join(CSRC, "kernels", "common.h")])
+
+
+def stream_tree_hash() -> str:
+    """Digest of everything _C_stream.so is built from."""
+    return _digest(stream_sources(), f"arch={ARCH};torch={torch_version()}")
+
+
+def library_hash(lib: str, symbol: str) -> str:
+    """The source digest compiled into a built library ('' when it is missing or has none)."""
+    import ctypes
+
+    if not os.path.exists(lib):
+        return ""
+    try:
+        f = getattr(ctypes.CDLL(lib, mode=getattr(os, "RTLD_LAZY", 1) | ctypes.RTLD_GLOBAL), symbol)
+    except (OSError, AttributeError):
+        return ""
+    f.restype = ctypes.c_char_p
+    return f().decode()
+
+
+def build_stream(force: bool = False, jobs: int = 8, log=None) -> str:
+    """The fp32-residual-stream kernels (csrc/stream/) -> ``_C_stream.so``
+    (torch.ops.akap_stream), a library of its own: a model that runs on these kernels alone
+    compiles and loads nothing else."""
+    log = log or BuildLog()
+    os.makedirs(BUILD, exist_ok=True)
+    inc, lib, abi = _torch_paths()
+    headers = [f for f in stream_sources() if f.endswith(".h")]
+    tv = torch_version()
+    common = ["-O3", "-std=c++17", "-fPIC", f"-D_GLIBCXX_USE_CXX11_ABI={abi}"]
+    todo, objs = [], []
+    for src in sorted(glob.glob(os.path.join(STREAM_SRC, "*.hip"))):
+        obj = os.path.join(BUILD, "stream_" + os.path.basename(src) + ".o")
+        objs.append(obj)
+        cmd = [HIPCC, f"--offload-arch={ARCH}", *common, *NO_PACKED_FP32, "-c", src, "-o", obj]
+        digest = _digest([src] + headers, " ".join(cmd[:-3]))
+        why = "forced" if force else _stale(obj, digest)
+        if why:
+            log(f"compile stream/{os.path.basename(src)} ({why})")
+            todo.append((cmd, obj, digest))
+    ops_src = os.path.join(STREAM_SRC, "stream_ops.cpp")
+    ops_obj = os.path.join(BUILD, "stream_ops.cpp.o")
+    objs.append(ops_obj)
+    incs = sum([["-I", i] for i in inc], [])
+    cmd = [HIPCC, *common, "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-DTORCH_EXTENSION_NAME=_C_stream", *incs, "-I", "/opt/rocm/include", "-x", "c++", "-c",
+           ops_src, "-o", ops_obj]
+    digest = _digest([ops_src] + headers, " ".join(cmd[:-3]) + f";torch={tv}")
+    why = "forced" if force else _stale(ops_obj, digest)
+    if why:
+        log(f"compile stream/stream_ops.cpp ({why})")
+        todo.append((cmd, ops_obj, digest))
+    with cf.ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
+        list(ex.map(_compile, todo))
+    out = os.path.join(PKG, "_C_stream.so")
+    tree = stream_tree_hash()
+    info_src = os.path.join(BUILD, "stream_build_info.c")
+    info_obj = info_src + ".o"
+    with open(info_src, "w") as f:
+        f.write(f'const char* akap_stream_build_hash(void) {{ return "{tree}"; }}\n')
+    _run(["gcc", "-O1", "-fPIC", "-c", info_src, "-o", info_obj])
+    link_digest = _digest(objs + [info_obj])
+    why = "forced" if force else ("objects rebuilt" if todo else _stale(out, link_digest))
+    if why:
+        log(f"link _C_stream.so ({why}); tree {tree[:16]}, torch {tv}")
+        tmp = out + f".tmp{os.getpid()}"
+        _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, info_obj, "-o", tmp,
+              f"-L{lib}", f"-Wl,-rpath,{lib}", "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu",
+              "-ltorch_hip", "-lamdhip64"])
+        os.replace(tmp, out)
+        with open(out + ".sha", "w") as f:
+            f.write(link_digest + "\n")
+    else:
+        log(f"reuse _C_stream.so: built from this tree ({tree[:16]}, torch {tv})")
     return out
 
 
@@ -227,6 +314,7 @@ def build(force: bool = False, jobs: int = 8) -> list[str]:
     build_runtime(force, log=log)
     build_pmc_tool(force, log=log)
     build_kernels(force, jobs, log=log)
+    build_stream(force, jobs, log=log)
     return log.lines
 
 

@@ -1,0 +1,212 @@
+// Row kernels of the fp32 residual stream: scaled embedding, residual update fused with the
+// next RMS norm, squared-ReLU, and the q/k whole-projection norm + rotary + paged-cache write.
+//
+// All memory-bound, one workgroup per token row; sums of squares, the norm scale, angles and
+// the residual sum are fp32 whatever the storage type.
+#include "../kernels/common.h"
+#include "stream.h"
+
+namespace akap_stream {
+
+using akap::bf16;
+using akap::block_sum;
+
+template <typename T>
+__device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
+template <typename T>
+__device__ __forceinline__ void stf(T* p, float v) { *p = (T)v; }
+
+template <typename T>
+__global__ __launch_bounds__(256) void embed_scaled_kernel(float* __restrict__ out,
+                                                           const int64_t* __restrict__ ids,
+                                                           const T* __restrict__ table, int d,
+                                                           int vocab, float scale) {
+  const int row = blockIdx.x;
+  const int64_t id = ids[row];
+  const bool ok = id >= 0 && id < vocab;
+  const T* src = table + (size_t)(ok ? id : 0) * d;
+  float* dst = out + (size_t)row * d;
+  for (int c = threadIdx.x; c < d; c += 256) dst[c] = ok ? ldf(src + c) * scale : 0.f;
+}
+
+void launch_embed_scaled(float* out, const int64_t* ids, const void* table, bool f32, int rows,
+                         int d, int vocab, float scale, hipStream_t s) {
+  if (rows <= 0) return;
+  if (f32)
+    embed_scaled_kernel<float><<<rows, 256, 0, s>>>(out, ids, (const float*)table, d, vocab, scale);
+  else
+    embed_scaled_kernel<bf16><<<rows, 256, 0, s>>>(out, ids, (const bf16*)table, d, vocab, scale);
+}
+
+// x += mult * y, out = x / sqrt(mean(x^2) + eps) * w.  The row stays in registers between the
+// two passes when it fits (d <= 256 * NR), so x is read and written once.
+template <typename TY, typename TO, int NR>
+__global__ __launch_bounds__(256) void add_norm_kernel(TO* __restrict__ out, float* __restrict__ x,
+                                                       const TY* __restrict__ y, int y_stride,
+                                                       float mult, const float* __restrict__ w,
+                                                       int d, int out_stride, float eps) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  float* xr = x + (size_t)row * d;
+  const TY* yr = y ? y + (size_t)row * y_stride : nullptr;
+  float v[NR];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    const int c = i * 256 + threadIdx.x;
+    v[i] = 0.f;
+    if (c < d) {
+      float f = xr[c];
+      if (yr) {
+        f += mult * ldf(yr + c);
+        xr[c] = f;
+      }
+      v[i] = f;
+      ss += f * f;
+    }
+  }
+  // rows wider than the register tile: the rest streams through memory twice
+  for (int c = NR * 256 + threadIdx.x; c < d; c += 256) {
+    float f = xr[c];
+    if (yr) {
+      f += mult * ldf(yr + c);
+      xr[c] = f;
+    }
+    ss += f * f;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+  TO* orow = out + (size_t)row * out_stride;
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    const int c = i * 256 + threadIdx.x;
+    if (c < d) stf(orow + c, v[i] * inv * w[c]);
+  }
+  for (int c = NR * 256 + threadIdx.x; c < d; c += 256) stf(orow + c, xr[c] * inv * w[c]);
+}
+
+template <typename TY, typename TO>
+static void add_norm_t(void* out, float* x, const void* y, int y_stride, float mult,
+                       const float* w, int rows, int d, int out_stride, float eps, hipStream_t s) {
+  if (d <= 1024)
+    add_norm_kernel<TY, TO, 4><<<rows, 256, 0, s>>>((TO*)out, x, (const TY*)y, y_stride, mult, w, d,
+                                                    out_stride, eps);
+  else
+    add_norm_kernel<TY, TO, 16><<<rows, 256, 0, s>>>((TO*)out, x, (const TY*)y, y_stride, mult, w,
+                                                     d, out_stride, eps);
+}
+
+void launch_add_norm(void* out, bool out_f32, float* x, const void* y, bool y_f32, int y_stride,
+                     float mult, const float* w, int rows, int d, int out_stride, float eps,
+                     hipStream_t s) {
+  if (rows <= 0) return;
+  if (out_f32 && y_f32)
+    add_norm_t<float, float>(out, x, y, y_stride, mult, w, rows, d, out_stride, eps, s);
+  else if (out_f32)
+    add_norm_t<bf16, float>(out, x, y, y_stride, mult, w, rows, d, out_stride, eps, s);
+  else if (y_f32)
+    add_norm_t<float, bf16>(out, x, y, y_stride, mult, w, rows, d, out_stride, eps, s);
+  else
+    add_norm_t<bf16, bf16>(out, x, y, y_stride, mult, w, rows, d, out_stride, eps, s);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void relu2_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                                    int F, int x_stride, int out_stride) {
+  const int row = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= F) return;
+  const float f = fmaxf(ldf(x + (size_t)row * x_stride + c), 0.f);
+  stf(out + (size_t)row * out_stride + c, f * f);
+}
+
+void launch_relu2(void* out, const void* x, bool f32, int rows, int F, int x_stride,
+                  int out_stride, hipStream_t s) {
+  if (rows <= 0 || F <= 0) return;
+  const dim3 grid((F + 255) / 256, rows);
+  if (f32)
+    relu2_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)x, F, x_stride, out_stride);
+  else
+    relu2_kernel<bf16><<<grid, 256, 0, s>>>((bf16*)out, (const bf16*)x, F, x_stride, out_stride);
+}
+
+// One workgroup per token: sums of squares over the WHOLE q and the WHOLE k projection, then
+// every thread norms, weights and rotates element pairs (2i, 2i+1) and stores q to q_out, k to
+// the K cache and the raw k to the V cache.
+template <typename T>
+__global__ __launch_bounds__(256) void proj_norm_rope_cache_kernel(ProjParams p) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const T* row = (const T*)p.proj + (size_t)t * p.proj_stride;
+  const T* qr = row + p.q_off;
+  const T* kr = row + p.k_off;
+  const int HD = p.H * p.D, GD = p.G * p.D;
+  float sq = 0.f, sk = 0.f;
+  for (int c = threadIdx.x; c < HD; c += 256) {
+    const float f = ldf(qr + c);
+    sq += f * f;
+  }
+  for (int c = threadIdx.x; c < GD; c += 256) {
+    const float f = ldf(kr + c);
+    sk += f * f;
+  }
+  sq = block_sum(sq, scratch);
+  sk = block_sum(sk, scratch);
+  const float iq = 1.0f / sqrtf(sq / (float)HD + p.eps);
+  const float ik = 1.0f / sqrtf(sk / (float)GD + p.eps);
+  int64_t pos = p.positions[t];
+  if (pos < 0) pos = 0;
+  if (pos >= p.max_pos) pos = p.max_pos - 1;  // (host checks the table covers the model length)
+  const float* cs = p.cos_sin ? p.cos_sin + (size_t)pos * p.rot_dims : nullptr;
+  const int half = p.D >> 1, rh = p.rot_dims >> 1;
+  T* qo = (T*)p.q_out + (size_t)t * HD;
+  for (int e = threadIdx.x; e < (HD >> 1); e += 256) {
+    const int i = e % half;
+    const int c = (e / half) * p.D + 2 * i;
+    float u = ldf(qr + c) * iq * p.q_w[c];
+    float v = ldf(qr + c + 1) * iq * p.q_w[c + 1];
+    if (cs && i < rh) {
+      const float co = cs[i], si = cs[rh + i];
+      const float ru = u * co - v * si;
+      v = v * co + u * si;
+      u = ru;
+    }
+    stf(qo + c, u);
+    stf(qo + c + 1, v);
+  }
+  const int64_t slot = p.slots[t];
+  if (slot < 0 || slot >= p.num_slots) return;
+  const int64_t blk = slot / p.BS;
+  const int off = (int)(slot % p.BS);
+  for (int e = threadIdx.x; e < (GD >> 1); e += 256) {
+    const int i = e % half;
+    const int g = e / half;
+    const int c = g * p.D + 2 * i;
+    const float ru = ldf(kr + c), rv = ldf(kr + c + 1);
+    float u = ru * ik * p.k_w[c];
+    float v = rv * ik * p.k_w[c + 1];
+    if (cs && i < rh) {
+      const float co = cs[i], si = cs[rh + i];
+      const float nu = u * co - v * si;
+      v = v * co + u * si;
+      u = nu;
+    }
+    const size_t o = (((size_t)blk * p.G + g) * p.BS + off) * p.D + 2 * i;
+    T* kc = (T*)p.k_cache + o;
+    T* vc = (T*)p.v_cache + o;
+    stf(kc, u);
+    stf(kc + 1, v);
+    vc[0] = kr[c];      // the values are the projected keys, untouched
+    vc[1] = kr[c + 1];
+  }
+}
+
+void launch_proj_norm_rope_cache(const ProjParams& p, bool f32, hipStream_t s) {
+  if (p.T <= 0) return;
+  if (f32)
+    proj_norm_rope_cache_kernel<float><<<p.T, 256, 0, s>>>(p);
+  else
+    proj_norm_rope_cache_kernel<bf16><<<p.T, 256, 0, s>>>(p);
+}
+
+}  // namespace akap_stream
