@@ -559,8 +559,7 @@ class ModelRunner:
         # (and not reused by later captures in the shared pool) while referenced here
         self._step_logits[n] = logits
         if not self.ecfg.logits_only:
-            self._sample(logits if logits.dtype == torch.bfloat16 or not self.is_gpu
-                         else logits.to(torch.bfloat16), n, extras, src=dd)
+            self._sample(logits, n, extras, src=dd)
         if self._ep_moe:
             moe_mod.ep_overflow_reduce(self.device)
 
