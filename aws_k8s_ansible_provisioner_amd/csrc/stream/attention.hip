@@ -1,16 +1,26 @@
 // Paged attention with a lower-bounded causal mask (chunks and / or a sliding window), a
-// per-head sink logit in the softmax denominator and a per-head sigmoid output gate, over
-// K / V caches [NB, G, BS, D] of bf16 or fp32 with any head size D.
+// per-head sink logit in the softmax denominator and a per-head sigmoid output gate, over a
+// K cache [NB, G, BS, D] and a V cache [NB, G, BS/8, D, 8] of bf16 or fp32.
 //
 // Scores, the running softmax and the gate are fp32.  A query at position i sees the keys
 // [lo(i), i] with lo(i) = max(floor(i / chunk) * chunk, i - window + 1, 0): only that range is
 // read, so a chunked layer costs O(chunk) per token however long the sequence.
 //
-// row kernel (any D, bf16 / fp32): one wave per (token, head).  Per 64-key piece each lane
-//   scores one key (q broadcast from LDS), the wave takes the piece's max and sum, and lanes
-//   then own output dimensions for the P.V update (coalesced V rows).  Prefill tiles give a
-//   workgroup's four waves the tokens of one tile; decode rows cut [lo, i] into partitions
-//   that a second launch merges together with the sink and the gate.
+// row kernel (any D <= 256, bf16 / fp32): one wave per (token, head).  Keys go in 64-aligned
+//   pieces: each lane scores one key (q broadcast from LDS, 16-byte K loads), the wave takes
+//   the piece's max and sum, and lanes then own output dimensions for the P.V update, reading
+//   V one 8-key group (16 bytes) at a time.  Decode rows cut [lo, i] into partitions that a
+//   second launch merges together with the sink and the gate; prefill tiles give a
+//   workgroup's four waves the tokens of one tile (fp32 models, head sizes the matrix kernel
+//   does not take).
+// matrix kernel (prefill, bf16, D in {32, 64, 128, 256}): one wave per 32 queries of a head,
+//   v_mfma_f32_32x32x16_bf16 for S^T = K Q^T and O^T = V^T P^T.  With keys as the MFMA rows,
+//   a query is a lane column: its softmax statistics are 16 registers and one cross-half
+//   exchange, never an LDS pass.  The A rows of the K fragment are loaded in the order that
+//   makes the S^T accumulator registers of a lane exactly the 8 keys of a V group, so P goes
+//   from accumulator to B operand without any lane movement, and the V^T operand is one
+//   16-byte load from the grouped V cache.  K / V fragments come straight from global memory
+//   (L1 / L2 hits across the workgroup's four waves and the heads of a GQA group).
 #include "../kernels/common.h"
 #include "stream.h"
 
@@ -30,31 +40,77 @@ struct Softmax {
   float acc[kMaxDV];
 };
 
-// Keys [j0, j1) of one sequence against one query held in `qs` (LDS, D floats, pre-scaled).
-// `ps`: 64 floats of LDS owned by this wave.
+// 8 consecutive values of one (group, dim) of the V cache, as floats
+__device__ __forceinline__ void ld_group(float (&v)[8], const bf16* p) {
+  const akap::bf16x8 x = *reinterpret_cast<const akap::bf16x8*>(p);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = (float)x[e];
+}
+__device__ __forceinline__ void ld_group(float (&v)[8], const float* p) {
+  const akap::f32x4 a = *reinterpret_cast<const akap::f32x4*>(p);
+  const akap::f32x4 b = *reinterpret_cast<const akap::f32x4*>(p + 4);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[e] = a[e];
+    v[4 + e] = b[e];
+  }
+}
+
+// q . k over D dims; 16-byte loads when the row allows (D % 8 == 0: rows are 16-byte aligned)
+__device__ __forceinline__ float dot_row(const float* qs, const bf16* kr, int D) {
+  float dot = 0.f;
+  int d = 0;
+  if ((D & 7) == 0) {
+    for (; d < D; d += 8) {
+      const akap::bf16x8 x = *reinterpret_cast<const akap::bf16x8*>(kr + d);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot += qs[d + e] * (float)x[e];
+    }
+    return dot;
+  }
+  for (; d < D; ++d) dot += qs[d] * (float)kr[d];
+  return dot;
+}
+__device__ __forceinline__ float dot_row(const float* qs, const float* kr, int D) {
+  float dot = 0.f;
+  int d = 0;
+  if ((D & 3) == 0) {
+    for (; d < D; d += 4) {
+      const akap::f32x4 x = *reinterpret_cast<const akap::f32x4*>(kr + d);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dot += qs[d + e] * x[e];
+    }
+    return dot;
+  }
+  for (; d < D; ++d) dot += qs[d] * kr[d];
+  return dot;
+}
+
+// Keys [lo, j1) of one sequence against one query held in `qs` (LDS, D floats, pre-scaled),
+// in pieces aligned to 64 keys (so a piece is 8 whole V groups).  `ps`: 64 floats of LDS owned
+// by this wave.  Every key below j1 is a cached position of the sequence (its block exists).
 template <typename T>
 __device__ __forceinline__ void attend_range(Softmax& st, const float* qs, float* ps,
                                              const T* __restrict__ kc, const T* __restrict__ vc,
                                              const int32_t* __restrict__ bt, int max_blocks, int NB,
-                                             int G, int g, int BS, int D, int j0, int j1) {
+                                             int G, int g, int BS, int D, int lo, int j1) {
   const int lane = threadIdx.x & 63;
-  for (int base = j0; base < j1; base += 64) {
+  const int NG = BS >> 3;
+  for (int base = lo & ~63; base < j1; base += 64) {
     const int j = base + lane;
-    const bool ok = j < j1;
-    int row = 0;  // row of this lane's key in the [NB * G * BS, D] view of the cache
+    const bool ok = j >= lo && j < j1;
+    int grow = 0;  // this lane's key's row in the [NB * G * BS/8] group view of the V cache
     float s = -INFINITY;
-    if (ok) {
+    if (j < j1) {
       const int bi = j / BS;
       int blk = bi < max_blocks ? bt[bi] : 0;
       if (blk < 0 || blk >= NB) blk = 0;
-      row = (blk * G + g) * BS + (j - bi * BS);
-      const T* kr = kc + (size_t)row * D;
-      float dot = 0.f;
-      for (int d = 0; d < D; ++d) dot += qs[d] * ldf(kr + d);
-      s = dot;
+      const int off = j - bi * BS;
+      grow = (blk * G + g) * NG + (off >> 3);
+      if (ok) s = dot_row(qs, kc + ((size_t)(blk * G + g) * BS + off) * D, D);
     }
     const float mt = wave_max(s);
-    const float mn = fmaxf(st.m, mt);
+    const float mn = fmaxf(st.m, mt);  // finite: a piece always holds a visible key
     const float corr = expf(st.m - mn);  // first piece: exp(-inf) = 0
     const float pj = ok ? expf(s - mn) : 0.f;
     st.l = st.l * corr + wave_sum(pj);
@@ -63,15 +119,22 @@ __device__ __forceinline__ void attend_range(Softmax& st, const float* qs, float
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int c = 0; c < kMaxDV; ++c) st.acc[c] *= corr;
-    const int n = min(64, j1 - base);
-    for (int jj = 0; jj < n; ++jj) {
-      const float pv = ps[jj];
-      const int r = __shfl(row, jj, 64);
-      const T* vr = vc + (size_t)r * D;
+    for (int gi = 0; gi < 8; ++gi) {
+      const int gb = base + gi * 8;
+      if (gb >= j1 || gb + 8 <= lo) continue;  // (wave-uniform) nothing visible in this group
+      const int gr = __shfl(grow, gi * 8, 64);
+      float pv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pv[e] = ps[gi * 8 + e];
 #pragma unroll
       for (int c = 0; c < kMaxDV; ++c) {
         const int d = c * 64 + lane;
-        if (d < D) st.acc[c] += pv * ldf(vr + d);
+        if (d < D) {
+          float v[8];
+          ld_group(v, vc + ((size_t)gr * D + d) * 8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) st.acc[c] += pv[e] * v[e];
+        }
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -168,11 +231,12 @@ __global__ __launch_bounds__(64) void sink_attn_decode_rows_kernel(AttnParams p)
   }
   const int pos = kv - 1;
   const int lo = lower_bound_of(pos, p.chunk, p.window);
-  const int n = pos + 1 - lo;
-  int per = (n + p.num_parts - 1) / p.num_parts;
+  // partitions are whole 64-aligned pieces of [lo & ~63, pos]
+  const int a0 = lo & ~63;
+  int per = (pos + 1 - a0 + p.num_parts - 1) / p.num_parts;
   per = (per + 63) & ~63;
-  const int j0 = lo + part * per;
-  const int j1 = min(pos + 1, j0 + per);
+  const int j0 = max(lo, a0 + part * per);
+  const int j1 = min(pos + 1, a0 + (part + 1) * per);
   const int g = h / (p.H / p.G);
   Softmax st;
   st.m = -INFINITY;
@@ -230,9 +294,143 @@ __global__ __launch_bounds__(64) void sink_attn_decode_merge_kernel(AttnParams p
   finish_row<T>(st, p, b, h);
 }
 
+// swap bits 2 and 3: the A-row order of the K fragment (see the file comment)
+__device__ __forceinline__ int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
+
+// grid (tiles, H), 4 waves of 32 queries each: tiles of 128 tokens
+template <int DB>
+__global__ __launch_bounds__(256) void sink_attn_prefill_mfma_kernel(AttnParams p) {
+  constexpr int D = 32 * DB, KS = D / 16;
+  using akap::bf16x8;
+  using akap::f32x16;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int col = lane & 31, hf = lane >> 5;
+  const int tile = blockIdx.x, h = blockIdx.y;
+  const int b = p.tile_seq[tile];
+  if (b < 0 || b >= p.B) return;
+  const int qs0 = p.q_start[b];
+  const int qlen = p.q_start[b + 1] - qs0;
+  const int kv = p.seq_lens[b];
+  const int rend = min(p.tile_row[tile] + p.tile_rows, qlen);
+  const int r0 = p.tile_row[tile] + wave * 32;
+  if (r0 >= rend || kv < qlen) return;
+  const int g = h / (p.H / p.G);
+  const int32_t* bt = p.block_tables + (size_t)b * p.max_blocks;
+  const int r = r0 + col;
+  const bool valid = r < rend;
+  const int t = qs0 + (valid ? r : r0);
+  const int pos = kv - qlen + r;                       // this lane's query
+  const int pos_last = kv - qlen + min(r0 + 31, rend - 1);
+  const int lo_w = lower_bound_of(kv - qlen + r0, p.chunk, p.window);
+  const int my_lo = valid ? lower_bound_of(pos, p.chunk, p.window) : 0x7fffffff;
+  bf16x8 qf[KS];
+  {
+    const bf16* qp = (const bf16*)p.q + ((size_t)t * p.H + h) * D + 8 * hf;
+#pragma unroll
+    for (int c = 0; c < KS; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qp + 16 * c);
+  }
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int dt = 0; dt < DB; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  const int NG = p.BS >> 3;
+  const int krow = swap23(col);
+  for (int j0 = lo_w & ~31; j0 <= pos_last; j0 += 32) {
+    const int bi = j0 / p.BS;
+    int blk = bi < p.max_blocks ? bt[bi] : 0;
+    if (blk < 0 || blk >= p.NB) blk = 0;
+    const int off0 = j0 - bi * p.BS;  // a multiple of 32: the 32 keys lie in one block
+    const bf16* kp = (const bf16*)p.k_cache +
+                     ((size_t)(blk * p.G + g) * p.BS + off0 + krow) * D + 8 * hf;
+    f32x16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+    for (int c = 0; c < KS; ++c)
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(kp + 16 * c),
+                                                  qf[c], s, 0, 0, 0);
+    // accumulator register i of this lane: key j0 + 16 (i >> 3) + 8 hf + (i & 7), query `col`
+    float sv[16];
+    float bmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = j0 + 16 * (i >> 3) + 8 * hf + (i & 7);
+      const bool vis = key <= pos && key >= my_lo;
+      sv[i] = vis ? s[i] * p.scale : -INFINITY;
+      bmax = fmaxf(bmax, sv[i]);
+    }
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    const float mn = fmaxf(m, bmax);
+    const float ms = mn == -INFINITY ? 0.f : mn;  // nothing visible yet: every exp below is 0
+    const float alpha = expf(m - ms);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      sv[i] = expf(sv[i] - ms);
+      psum += sv[i];
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * alpha + psum;
+    m = mn;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) pb[i >> 3][i & 7] = (bf16)sv[i];
+    const bf16* vp = (const bf16*)p.v_cache +
+                     (((size_t)(blk * p.G + g) * NG + (off0 >> 3) + hf) * D + col) * 8;
+#pragma unroll
+    for (int dt = 0; dt < DB; ++dt) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl)
+        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            *reinterpret_cast<const bf16x8*>(vp + ((size_t)(2 * sl) * D + 32 * dt) * 8), pb[sl],
+            oacc[dt], 0, 0, 0);
+    }
+  }
+  if (!valid) return;
+  float corr = 1.f;
+  if (p.sink) {
+    const float sk = p.sink[h];
+    const float mf = fmaxf(m, sk);
+    corr = expf(m - mf);
+    l = l * corr + expf(sk - mf);
+  }
+  float gate = 1.f;
+  if (p.gate) {
+    const float z = (float)((const bf16*)p.gate)[(size_t)t * p.gate_stride + h];
+    gate = 1.0f / (1.0f + expf(-z));
+  }
+  const float f = l > 0.f ? corr * gate / l : 0.f;
+  // accumulator register i of oacc[dt]: dimension 32 dt + 8 (i >> 2) + 4 hf + (i & 3)
+  bf16* o = (bf16*)p.out + (size_t)t * p.out_stride + h * D;
+#pragma unroll
+  for (int dt = 0; dt < DB; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      o[32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = (bf16)(oacc[dt][i] * f);
+}
+
+// the matrix kernel takes bf16, these head sizes, and tiles of whole 32-query wave rows
+bool prefill_mfma_ok(const AttnParams& p, bool f32) {
+  return !f32 && (p.D == 32 || p.D == 64 || p.D == 128 || p.D == 256) && p.tile_rows == 128 &&
+         p.BS % 32 == 0;
+}
+
 void launch_sink_attention_prefill(const AttnParams& p, bool f32, hipStream_t s) {
   if (p.num_tiles <= 0) return;
   const dim3 grid(p.num_tiles, p.H);
+  if (prefill_mfma_ok(p, f32)) {
+    switch (p.D) {
+      case 32: sink_attn_prefill_mfma_kernel<1><<<grid, 256, 0, s>>>(p); break;
+      case 64: sink_attn_prefill_mfma_kernel<2><<<grid, 256, 0, s>>>(p); break;
+      case 128: sink_attn_prefill_mfma_kernel<4><<<grid, 256, 0, s>>>(p); break;
+      default: sink_attn_prefill_mfma_kernel<8><<<grid, 256, 0, s>>>(p); break;
+    }
+    return;
+  }
   const size_t sm = 4 * (p.D + 64) * sizeof(float);
   if (f32)
     sink_attn_prefill_rows_kernel<float><<<grid, 256, sm, s>>>(p);

@@ -191,13 +191,14 @@ __global__ __launch_bounds__(256) void proj_norm_rope_cache_kernel(ProjParams p)
       v = v * co + u * si;
       u = nu;
     }
-    const size_t o = (((size_t)blk * p.G + g) * p.BS + off) * p.D + 2 * i;
-    T* kc = (T*)p.k_cache + o;
-    T* vc = (T*)p.v_cache + o;
+    T* kc = (T*)p.k_cache + (((size_t)blk * p.G + g) * p.BS + off) * p.D + 2 * i;
     stf(kc, u);
     stf(kc + 1, v);
-    vc[0] = kr[c];      // the values are the projected keys, untouched
-    vc[1] = kr[c + 1];
+    // the values are the projected keys, untouched; V cache [NB, G, BS/8, D, 8]
+    T* vc = (T*)p.v_cache +
+            ((((size_t)blk * p.G + g) * (p.BS >> 3) + (off >> 3)) * p.D + 2 * i) * 8 + (off & 7);
+    vc[0] = kr[c];
+    vc[8] = kr[c + 1];
   }
 }
 

@@ -73,10 +73,13 @@ void relu2(Tensor out, Tensor x) {
 
 void check_cache(const Tensor& k_cache, const Tensor& v_cache, int64_t G, int64_t D) {
   CHECK_GPU(k_cache); CHECK_GPU(v_cache); CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
-  TORCH_CHECK(k_cache.dim() == 4 && k_cache.sizes() == v_cache.sizes() &&
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 5 &&
                   k_cache.scalar_type() == v_cache.scalar_type(),
-              "K and V caches must be equal-shaped [NB, G, BS, D]");
+              "caches must be K [NB, G, BS, D] and V [NB, G, BS/8, D, 8]");
   TORCH_CHECK(k_cache.size(1) == G && k_cache.size(3) == D, "cache does not match G / D");
+  TORCH_CHECK(k_cache.size(2) % 8 == 0 && v_cache.size(0) == k_cache.size(0) &&
+                  v_cache.size(1) == G && v_cache.size(2) * 8 == k_cache.size(2) &&
+                  v_cache.size(3) == D && v_cache.size(4) == 8, "V cache does not match K cache");
   TORCH_CHECK(k_cache.size(0) * G * k_cache.size(2) < (1LL << 31), "cache has too many rows");
 }
 

@@ -32,7 +32,7 @@ from .config import LayeredConfig, LayerSpec
 from .transformer import AttnBatch
 
 # tokens per tile of the prefill attention map (csrc/stream/attention.hip: one workgroup)
-PREFILL_TILE_TOKENS = 64
+PREFILL_TILE_TOKENS = 128
 
 
 @dataclasses.dataclass
@@ -211,7 +211,8 @@ class BidetarLM:
     def allocate_kv_segments(self, num_blocks: int, block_size: int, kv_dtype: str = "auto",
                              max_segment_bytes: Optional[int] = None) -> list:
         """One allocation [2, NB, G, BS, D] per layer RUN (a looped layer has a cache per
-        pass; layers may differ in G and D), zero-filled, in the model's dtype."""
+        pass; layers may differ in G and D), zero-filled, in the model's dtype.  Plane 0 is K
+        (token-major), plane 1 the same bytes viewed as V's [NB, G, BS/8, D, 8] groups."""
         if kv_dtype not in ("auto", "bf16", "bfloat16"):
             raise ValueError("Bidetar: the KV cache is kept in the model's dtype (no fp8)")
         segs = []
@@ -226,7 +227,8 @@ class BidetarLM:
 
     def cache_views(self, kv, block_size: int):
         segs = list(kv)
-        return [s[0] for s in segs], [s[1] for s in segs]
+        return [s[0] for s in segs], [s[1].view(s.shape[1], s.shape[2], s.shape[3] // 8, s.shape[4], 8)
+                                      for s in segs]
 
     # ------------------------------------------------------------------ forward
     def _decode_parts(self, rows: int, m) -> int:

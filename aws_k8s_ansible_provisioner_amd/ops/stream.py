@@ -6,7 +6,9 @@ kernels are templated on the activation type (bf16 or fp32) and take every size 
 (any head size, head count and GQA ratio), so a model's weights and KV cache may be bf16 or
 fp32; norms, rotary angles, attention scores and weights and the residual sum are fp32 in both.
 
-KV cache layout of these ops: K and V [num_blocks, G, block_size, D], token-major rows.
+KV cache layout of these ops: K [num_blocks, G, block_size, D] (token-major rows) and
+V [num_blocks, G, block_size / 8, D, 8] (groups of 8 tokens, dimension-major inside a group: the
+8 keys a matrix-core operand contracts over, or a decode lane accumulates, are one 16-byte load).
 """
 from __future__ import annotations
 
@@ -132,7 +134,7 @@ def proj_norm_rope_cache(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch
     cos_sin.shape[1] dimensions, interleaved pairs (2i, 2i+1), by the angle row of
     positions[t].  q goes to q_out [T, H, D]; k to k_cache at slots[t]; the raw k (before norm
     and rotation) to v_cache at the same slot: the values are the keys' projection.  Slot -1
-    writes nothing.  Caches are [NB, G, BS, D]."""
+    writes nothing.  k_cache [NB, G, BS, D], v_cache [NB, G, BS/8, D, 8]."""
     if _native(proj):
         torch.ops.akap_stream.proj_norm_rope_cache(proj, q_out, k_cache, v_cache, positions, slots,
                                                    cos_sin, q_w, k_w, H, G, D, q_off, k_off,
@@ -161,7 +163,19 @@ def proj_norm_rope_cache(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch
     ok = slots >= 0
     sl = slots[ok].long()
     k_cache[sl // BS, :, sl % BS] = kn[ok].to(k_cache.dtype)
-    v_cache[sl // BS, :, sl % BS] = k.view(T, G, D)[ok].to(v_cache.dtype)
+    v_cache[sl // BS, :, (sl % BS) // 8, :, sl % 8] = k.view(T, G, D)[ok].to(v_cache.dtype)
+
+
+def v_tokens(v_cache: torch.Tensor) -> torch.Tensor:
+    """The V cache [NB, G, BS/8, D, 8] as token-major rows [NB, G, BS, D] (a copy)."""
+    NB, G, NG, D, _ = v_cache.shape
+    return v_cache.permute(0, 1, 2, 4, 3).reshape(NB, G, NG * 8, D)
+
+
+def v_from_tokens(v: torch.Tensor) -> torch.Tensor:
+    """Token-major values [NB, G, BS, D] in the V cache layout [NB, G, BS/8, D, 8]."""
+    NB, G, BS, D = v.shape
+    return v.view(NB, G, BS // 8, 8, D).permute(0, 1, 2, 4, 3).contiguous()
 
 
 # ----------------------------------------------------------------------------- attention
@@ -174,7 +188,7 @@ def _attend_rows(out, q, k_cache, v_cache, bt_row, kv_len: int, pos0: int, rows:
     nb = -(-kv_len // BS)
     blocks = bt_row[:nb].long()
     K = k_cache[blocks].permute(1, 0, 2, 3).reshape(G, nb * BS, D)[:, :kv_len].float()
-    V = v_cache[blocks].permute(1, 0, 2, 3).reshape(G, nb * BS, D)[:, :kv_len].float()
+    V = v_tokens(v_cache[blocks]).permute(1, 0, 2, 3).reshape(G, nb * BS, D)[:, :kv_len].float()
     i = torch.arange(pos0, pos0 + n)[:, None]
     j = torch.arange(kv_len)[None, :]
     ok = j <= i

@@ -108,11 +108,12 @@ def test_projection_norm_rotation_and_value_cache():
     slots = torch.tensor([3, 0, 9, 31, 32, 63, 12, 40, -1])
     rot = {"dims": R, "base": 20.0, "scaling": None}
     q = torch.zeros(T, H, D)
-    kc, vc = torch.zeros(NB, G, BS, D), torch.zeros(NB, G, BS, D)
+    kc, vc = torch.zeros(NB, G, BS, D), torch.zeros(NB, G, BS // 8, D, 8)
     sops.proj_norm_rope_cache(proj, q, kc, vc, pos, slots, sops.rotary_table(64, R, 20.0), qw, kw,
                               H, G, D, 5, 5 + H * D, 1e-5)
     f = oracle.rotary_frequencies(rot)
     p64 = proj.double()
+    vc = sops.v_tokens(vc)  # the V cache keeps 8-token groups; compare token-major
     for t in range(T):
         qn = (oracle.rms_unit(p64[t, 5:5 + H * D], 1e-5) * qw.double()).reshape(H, D)
         kraw = p64[t, 5 + H * D:].reshape(G, D)
@@ -145,7 +146,7 @@ def spike_case(chunk, n, q_pos, key_pos, BS=32):
     q[0, 0, 0] = 30.0
     kc[bt[0, key_pos // BS], 0, key_pos % BS, 0] = 30.0
     vc[bt[0, key_pos // BS], 0, key_pos % BS, :] = 1.0
-    return q, kc, vc, bt
+    return q, kc, sops.v_from_tokens(vc), bt
 
 
 @pytest.mark.parametrize("chunk,n,q_pos,key_pos,seen", [
@@ -186,7 +187,7 @@ def test_sink_counts_once_unscaled_and_gate():
     scale; the gate multiplies the head's output by sigmoid(z)."""
     n, D, BS = 5, 4, 32
     kc = torch.zeros(1, 1, BS, D)
-    vc = torch.ones(1, 1, BS, D)
+    vc = torch.ones(1, 1, BS // 8, D, 8)
     q = torch.zeros(1, 2, D)
     bt = torch.zeros(1, 1, dtype=torch.int32)
     sink = torch.tensor([math.log(3.0), -40.0])

@@ -55,7 +55,7 @@ def paged(B, lens, BS, G, D, dt, g, extra_blocks=3):
         bt[b, :nb] = perm[o:o + nb].int()
         o += nb
     kc = torch.randn(NB, G, BS, D, generator=g).to(dt)
-    vc = torch.randn(NB, G, BS, D, generator=g).to(dt)
+    vc = sops.v_from_tokens(torch.randn(NB, G, BS, D, generator=g)).to(dt)
     return kc, vc, bt
 
 
@@ -78,7 +78,7 @@ def test_proj_norm_rope_cache(dt, H, G, D, rd):
     def run(dev):
         q = torch.zeros(T, H, D, dtype=dt, device=dev)
         kc = torch.zeros(NB, G, BS, D, dtype=dt, device=dev)
-        vc = torch.zeros(NB, G, BS, D, dtype=dt, device=dev)
+        vc = torch.zeros(NB, G, BS // 8, D, 8, dtype=dt, device=dev)
         sops.proj_norm_rope_cache(proj.to(dev), q, kc, vc, pos.to(dev), slots.to(dev), cs.to(dev),
                                   qw.to(dev), kw.to(dev), H, G, D, 8, 8 + H * D, 1e-5)
         return q.cpu().float(), kc.cpu().float(), vc.cpu().float()
@@ -99,8 +99,9 @@ CASES = [  # H, G, D, chunk, window, sink, gate
 
 
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("tr", [64, 128])   # 128-token tiles in bf16: the matrix-core kernel
 @pytest.mark.parametrize("H,G,D,chunk,window,use_sink,use_gate", CASES)
-def test_sink_attention_prefill(dt, H, G, D, chunk, window, use_sink, use_gate):
+def test_sink_attention_prefill(dt, tr, H, G, D, chunk, window, use_sink, use_gate):
     g = torch.Generator().manual_seed(H + D + chunk + window)
     BS = 32
     lens = [700, 130, 65, 1, 257]       # cached tokens after the step
@@ -112,7 +113,6 @@ def test_sink_attention_prefill(dt, H, G, D, chunk, window, use_sink, use_gate):
     gate = torch.randn(T, H + 3, generator=g).to(dt)[:, 1:1 + H] if use_gate else None
     sink = torch.randn(H, generator=g) if use_sink else None
     qs = torch.tensor([0] + list(torch.tensor(qlens).cumsum(0)), dtype=torch.int32)
-    tr = 64
     ts, trow = [], []
     for b, n in enumerate(qlens):
         for r in range(0, n, tr):
