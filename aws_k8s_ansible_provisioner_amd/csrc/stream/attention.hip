@@ -13,8 +13,10 @@
 //   second launch merges together with the sink and the gate; prefill tiles give a
 //   workgroup's four waves the tokens of one tile (fp32 models, head sizes the matrix kernel
 //   does not take).
-// matrix kernel (prefill, bf16, D in {32, 64, 128, 256}): one wave per 32 queries of a head,
-//   v_mfma_f32_32x32x16_bf16 for S^T = K Q^T and O^T = V^T P^T.  With keys as the MFMA rows,
+// matrix kernels (bf16, D in {32, 64, 128, 256}): v_mfma_f32_32x32x16_bf16 for S^T = K Q^T and
+//   O^T = V^T P^T.  Prefill: one wave per 64 queries of a head (two 32-column tiles share every
+//   K / V fragment load).  Decode: the columns of a tile are the query heads of one K/V head,
+//   so a GQA group reads its keys and values once; the key range is split over workgroups.  With keys as the MFMA rows,
 //   a query is a lane column: its softmax statistics are 16 registers and one cross-half
 //   exchange, never an LDS pass.  The A rows of the K fragment are loaded in the order that
 //   makes the S^T accumulator registers of a lane exactly the 8 keys of a V group, so P goes
@@ -297,12 +299,143 @@ __global__ __launch_bounds__(64) void sink_attn_decode_merge_kernel(AttnParams p
 // swap bits 2 and 3: the A-row order of the K fragment (see the file comment)
 __device__ __forceinline__ int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
 
-// grid (tiles, H), 4 waves of 32 queries each: tiles of 128 tokens
-template <int DB>
-__global__ __launch_bounds__(256) void sink_attn_prefill_mfma_kernel(AttnParams p) {
-  constexpr int D = 32 * DB, KS = D / 16;
+// Running state of NQ tiles of 32 query columns (one column per lane & 31, both lane halves):
+// O^T accumulators [D / 32 blocks][16 registers], softmax max and sum per column.
+template <int DB, int NQ>
+struct MfmaState {
+  akap::f32x16 o[NQ][DB];
+  float m[NQ], l[NQ];
+};
+
+// Keys [jb, je] (jb a multiple of 32) against the wave's query columns.  qf: the columns' Q
+// fragments (B operands); pos / my_lo: each lane's query position and lowest visible key per
+// tile (my_lo > pos: an unused column).  Each K and V fragment is loaded once, straight from
+// the cache, and feeds the MFMAs of all NQ tiles.
+template <int DB, int NQ>
+__device__ __forceinline__ void mfma_attend(MfmaState<DB, NQ>& st, const AttnParams& p,
+                                            const int32_t* __restrict__ bt, int g,
+                                            const akap::bf16x8 (&qf)[NQ][2 * DB],
+                                            const int (&pos)[NQ], const int (&my_lo)[NQ], int jb,
+                                            int je) {
+  constexpr int D = 32 * DB, KS = 2 * DB;
   using akap::bf16x8;
   using akap::f32x16;
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 31, hf = lane >> 5;
+  const int NG = p.BS >> 3;
+  const int krow = swap23(col);
+  for (int j0 = jb; j0 <= je; j0 += 32) {
+    const int bi = j0 / p.BS;
+    int blk = bi < p.max_blocks ? bt[bi] : 0;
+    if (blk < 0 || blk >= p.NB) blk = 0;
+    const int off0 = j0 - bi * p.BS;  // a multiple of 32: the 32 keys lie in one block
+    const bf16* kp = (const bf16*)p.k_cache +
+                     ((size_t)(blk * p.G + g) * p.BS + off0 + krow) * D + 8 * hf;
+    const bf16* vp = (const bf16*)p.v_cache +
+                     (((size_t)(blk * p.G + g) * NG + (off0 >> 3) + hf) * D + col) * 8;
+    bf16x8 kf[KS];
+#pragma unroll
+    for (int c = 0; c < KS; ++c) kf[c] = *reinterpret_cast<const bf16x8*>(kp + 16 * c);
+    bf16x8 pb[NQ][2];
+    float alpha[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      f32x16 s;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+      for (int c = 0; c < KS; ++c)
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[c], qf[q][c], s, 0, 0, 0);
+      // accumulator register i of this lane: key j0 + 16 (i >> 3) + 8 hf + (i & 7), column col
+      float sv[16];
+      float bmax = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = j0 + 16 * (i >> 3) + 8 * hf + (i & 7);
+        const bool vis = key <= pos[q] && key >= my_lo[q];
+        sv[i] = vis ? s[i] * p.scale : -INFINITY;
+        bmax = fmaxf(bmax, sv[i]);
+      }
+      bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+      const float mn = fmaxf(st.m[q], bmax);
+      const float ms = mn == -INFINITY ? 0.f : mn;  // nothing visible yet: every exp below is 0
+      alpha[q] = __expf(st.m[q] - ms);
+      float psum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        sv[i] = __expf(sv[i] - ms);
+        psum += sv[i];
+      }
+      psum += __shfl_xor(psum, 32, 64);
+      st.l[q] = st.l[q] * alpha[q] + psum;
+      st.m[q] = mn;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) pb[q][i >> 3][i & 7] = (bf16)sv[i];
+    }
+#pragma unroll
+    for (int dt = 0; dt < DB; ++dt) {
+#pragma unroll
+      for (int q = 0; q < NQ; ++q)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) st.o[q][dt][i] *= alpha[q];
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl) {
+        const bf16x8 vf =
+            *reinterpret_cast<const bf16x8*>(vp + ((size_t)(2 * sl) * D + 32 * dt) * 8);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q)
+          st.o[q][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[q][sl], st.o[q][dt], 0, 0, 0);
+      }
+    }
+  }
+}
+
+template <int DB, int NQ>
+__device__ __forceinline__ void mfma_init(MfmaState<DB, NQ>& st) {
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    st.m[q] = -INFINITY;
+    st.l[q] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DB; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) st.o[q][dt][i] = 0.f;
+  }
+}
+
+// sink, normalise, gate and store column tile q of a lane (token row t, head h).
+// Accumulator register i of o[dt]: dimension 32 dt + 8 (i >> 2) + 4 hf + (i & 3).
+template <int DB, int NQ>
+__device__ __forceinline__ void mfma_finish(const MfmaState<DB, NQ>& st, int q,
+                                            const AttnParams& p, int t, int h) {
+  constexpr int D = 32 * DB;
+  const int hf = (threadIdx.x & 63) >> 5;
+  float l = st.l[q], corr = 1.f;
+  if (p.sink) {
+    const float sk = p.sink[h];
+    const float mf = fmaxf(st.m[q], sk);
+    corr = expf(st.m[q] - mf);
+    l = l * corr + expf(sk - mf);
+  }
+  float gate = 1.f;
+  if (p.gate) {
+    const float z = (float)((const bf16*)p.gate)[(size_t)t * p.gate_stride + h];
+    gate = 1.0f / (1.0f + expf(-z));
+  }
+  const float f = l > 0.f ? corr * gate / l : 0.f;
+  bf16* o = (bf16*)p.out + (size_t)t * p.out_stride + h * D;
+#pragma unroll
+  for (int dt = 0; dt < DB; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      o[32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = (bf16)(st.o[q][dt][i] * f);
+}
+
+// Prefill: grid (tiles of 128 tokens, H), 2 waves of 64 queries (two column tiles) each.
+template <int DB>
+__global__ __launch_bounds__(128) void sink_attn_prefill_mfma_kernel(AttnParams p) {
+  constexpr int D = 32 * DB, KS = 2 * DB, NQ = 2;
+  using akap::bf16x8;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int col = lane & 31, hf = lane >> 5;
   const int tile = blockIdx.x, h = blockIdx.y;
@@ -312,122 +445,105 @@ __global__ __launch_bounds__(256) void sink_attn_prefill_mfma_kernel(AttnParams 
   const int qlen = p.q_start[b + 1] - qs0;
   const int kv = p.seq_lens[b];
   const int rend = min(p.tile_row[tile] + p.tile_rows, qlen);
-  const int r0 = p.tile_row[tile] + wave * 32;
+  const int r0 = p.tile_row[tile] + wave * 64;
   if (r0 >= rend || kv < qlen) return;
   const int g = h / (p.H / p.G);
   const int32_t* bt = p.block_tables + (size_t)b * p.max_blocks;
-  const int r = r0 + col;
-  const bool valid = r < rend;
-  const int t = qs0 + (valid ? r : r0);
-  const int pos = kv - qlen + r;                       // this lane's query
-  const int pos_last = kv - qlen + min(r0 + 31, rend - 1);
+  int pos[NQ], my_lo[NQ], t[NQ];
+  bool valid[NQ];
+  bf16x8 qf[NQ][KS];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    const int r = r0 + 32 * q + col;
+    valid[q] = r < rend;
+    t[q] = qs0 + (valid[q] ? r : r0);
+    pos[q] = kv - qlen + r;
+    my_lo[q] = valid[q] ? lower_bound_of(pos[q], p.chunk, p.window) : 0x7fffffff;
+    const bf16* qp = (const bf16*)p.q + ((size_t)t[q] * p.H + h) * D + 8 * hf;
+#pragma unroll
+    for (int c = 0; c < KS; ++c) qf[q][c] = *reinterpret_cast<const bf16x8*>(qp + 16 * c);
+  }
+  const int pos_last = kv - qlen + min(r0 + 63, rend - 1);
   const int lo_w = lower_bound_of(kv - qlen + r0, p.chunk, p.window);
-  const int my_lo = valid ? lower_bound_of(pos, p.chunk, p.window) : 0x7fffffff;
-  bf16x8 qf[KS];
+  MfmaState<DB, NQ> st;
+  mfma_init(st);
+  mfma_attend<DB, NQ>(st, p, bt, g, qf, pos, my_lo, lo_w & ~31, pos_last);
+#pragma unroll
+  for (int q = 0; q < NQ; ++q)
+    if (valid[q]) mfma_finish<DB, NQ>(st, q, p, t[q], h);
+}
+
+// Decode: grid (B, G * ceil(rep / 32), parts), one wave: the query heads of one K/V head are
+// the columns of one tile, so K and V are read once per K/V head, not once per query head.
+template <int DB>
+__global__ __launch_bounds__(64) void sink_attn_decode_mfma_kernel(AttnParams p) {
+  constexpr int D = 32 * DB, KS = 2 * DB;
+  using akap::bf16x8;
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 31, hf = lane >> 5;
+  const int rep = p.H / p.G;
+  const int cgroups = (rep + 31) >> 5;
+  const int b = blockIdx.x, g = blockIdx.y / cgroups, part = blockIdx.z;
+  const int c0 = (blockIdx.y % cgroups) * 32;
+  const int kv = p.seq_lens[b];
+  const bool valid = c0 + col < rep;
+  const int h = g * rep + (valid ? c0 + col : 0);
+  if (kv <= 0) {  // padding row of a bucketed batch: defined output, no cache reads
+    if (part == 0 && valid) {
+      bf16* o = (bf16*)p.out + (size_t)b * p.out_stride + h * D;
+      for (int d = hf; d < D; d += 2) o[d] = (bf16)0.f;
+    }
+    return;
+  }
+  const int pos1 = kv - 1;
+  const int lo = lower_bound_of(pos1, p.chunk, p.window);
+  const int a0 = lo & ~31;
+  int per = (pos1 + 1 - a0 + p.num_parts - 1) / p.num_parts;
+  per = (per + 31) & ~31;
+  const int jb = a0 + part * per;
+  const int je = min(pos1, jb + per - 1);
+  int pos[1] = {pos1}, my_lo[1] = {valid ? lo : 0x7fffffff};
+  bf16x8 qf[1][KS];
   {
-    const bf16* qp = (const bf16*)p.q + ((size_t)t * p.H + h) * D + 8 * hf;
+    const bf16* qp = (const bf16*)p.q + ((size_t)b * p.H + h) * D + 8 * hf;
 #pragma unroll
-    for (int c = 0; c < KS; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qp + 16 * c);
+    for (int c = 0; c < KS; ++c) qf[0][c] = *reinterpret_cast<const bf16x8*>(qp + 16 * c);
   }
-  f32x16 oacc[DB];
-#pragma unroll
-  for (int dt = 0; dt < DB; ++dt)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
-  float m = -INFINITY, l = 0.f;
-  const int NG = p.BS >> 3;
-  const int krow = swap23(col);
-  for (int j0 = lo_w & ~31; j0 <= pos_last; j0 += 32) {
-    const int bi = j0 / p.BS;
-    int blk = bi < p.max_blocks ? bt[bi] : 0;
-    if (blk < 0 || blk >= p.NB) blk = 0;
-    const int off0 = j0 - bi * p.BS;  // a multiple of 32: the 32 keys lie in one block
-    const bf16* kp = (const bf16*)p.k_cache +
-                     ((size_t)(blk * p.G + g) * p.BS + off0 + krow) * D + 8 * hf;
-    f32x16 s;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) s[i] = 0.f;
-#pragma unroll
-    for (int c = 0; c < KS; ++c)
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(kp + 16 * c),
-                                                  qf[c], s, 0, 0, 0);
-    // accumulator register i of this lane: key j0 + 16 (i >> 3) + 8 hf + (i & 7), query `col`
-    float sv[16];
-    float bmax = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = j0 + 16 * (i >> 3) + 8 * hf + (i & 7);
-      const bool vis = key <= pos && key >= my_lo;
-      sv[i] = vis ? s[i] * p.scale : -INFINITY;
-      bmax = fmaxf(bmax, sv[i]);
-    }
-    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
-    const float mn = fmaxf(m, bmax);
-    const float ms = mn == -INFINITY ? 0.f : mn;  // nothing visible yet: every exp below is 0
-    const float alpha = expf(m - ms);
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      sv[i] = expf(sv[i] - ms);
-      psum += sv[i];
-    }
-    psum += __shfl_xor(psum, 32, 64);
-    l = l * alpha + psum;
-    m = mn;
-    bf16x8 pb[2];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) pb[i >> 3][i & 7] = (bf16)sv[i];
-    const bf16* vp = (const bf16*)p.v_cache +
-                     (((size_t)(blk * p.G + g) * NG + (off0 >> 3) + hf) * D + col) * 8;
-#pragma unroll
-    for (int dt = 0; dt < DB; ++dt) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
-#pragma unroll
-      for (int sl = 0; sl < 2; ++sl)
-        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            *reinterpret_cast<const bf16x8*>(vp + ((size_t)(2 * sl) * D + 32 * dt) * 8), pb[sl],
-            oacc[dt], 0, 0, 0);
-    }
-  }
+  MfmaState<DB, 1> st;
+  mfma_init(st);
+  if (jb <= je)
+    mfma_attend<DB, 1>(st, p, p.block_tables + (size_t)b * p.max_blocks, g, qf, pos, my_lo, jb, je);
   if (!valid) return;
-  float corr = 1.f;
-  if (p.sink) {
-    const float sk = p.sink[h];
-    const float mf = fmaxf(m, sk);
-    corr = expf(m - mf);
-    l = l * corr + expf(sk - mf);
+  if (p.num_parts == 1) {
+    mfma_finish<DB, 1>(st, 0, p, b, h);
+    return;
   }
-  float gate = 1.f;
-  if (p.gate) {
-    const float z = (float)((const bf16*)p.gate)[(size_t)t * p.gate_stride + h];
-    gate = 1.0f / (1.0f + expf(-z));
+  const size_t slot = ((size_t)b * p.H + h) * p.num_parts + part;
+  if (hf == 0) {
+    p.ws_ml[slot * 2] = st.m[0];
+    p.ws_ml[slot * 2 + 1] = st.l[0];
   }
-  const float f = l > 0.f ? corr * gate / l : 0.f;
-  // accumulator register i of oacc[dt]: dimension 32 dt + 8 (i >> 2) + 4 hf + (i & 3)
-  bf16* o = (bf16*)p.out + (size_t)t * p.out_stride + h * D;
 #pragma unroll
   for (int dt = 0; dt < DB; ++dt)
 #pragma unroll
     for (int i = 0; i < 16; ++i)
-      o[32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = (bf16)(oacc[dt][i] * f);
+      p.ws_o[slot * D + 32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = st.o[0][dt][i];
 }
 
-// the matrix kernel takes bf16, these head sizes, and tiles of whole 32-query wave rows
-bool prefill_mfma_ok(const AttnParams& p, bool f32) {
-  return !f32 && (p.D == 32 || p.D == 64 || p.D == 128 || p.D == 256) && p.tile_rows == 128 &&
-         p.BS % 32 == 0;
+// the matrix kernels take bf16 and these head sizes (prefill: tiles of 128 tokens)
+static bool mfma_ok(const AttnParams& p, bool f32) {
+  return !f32 && (p.D == 32 || p.D == 64 || p.D == 128 || p.D == 256) && p.BS % 32 == 0;
 }
 
 void launch_sink_attention_prefill(const AttnParams& p, bool f32, hipStream_t s) {
   if (p.num_tiles <= 0) return;
   const dim3 grid(p.num_tiles, p.H);
-  if (prefill_mfma_ok(p, f32)) {
+  if (mfma_ok(p, f32) && p.tile_rows == 128) {
     switch (p.D) {
-      case 32: sink_attn_prefill_mfma_kernel<1><<<grid, 256, 0, s>>>(p); break;
-      case 64: sink_attn_prefill_mfma_kernel<2><<<grid, 256, 0, s>>>(p); break;
-      case 128: sink_attn_prefill_mfma_kernel<4><<<grid, 256, 0, s>>>(p); break;
-      default: sink_attn_prefill_mfma_kernel<8><<<grid, 256, 0, s>>>(p); break;
+      case 32: sink_attn_prefill_mfma_kernel<1><<<grid, 128, 0, s>>>(p); break;
+      case 64: sink_attn_prefill_mfma_kernel<2><<<grid, 128, 0, s>>>(p); break;
+      case 128: sink_attn_prefill_mfma_kernel<4><<<grid, 128, 0, s>>>(p); break;
+      default: sink_attn_prefill_mfma_kernel<8><<<grid, 128, 0, s>>>(p); break;
     }
     return;
   }
@@ -442,7 +558,16 @@ void launch_sink_attention_decode(const AttnParams& p, bool f32, hipStream_t s) 
   if (p.B <= 0) return;
   const dim3 grid(p.B, p.H, p.num_parts);
   const size_t sm = (p.D + 64) * sizeof(float);
-  if (f32)
+  if (mfma_ok(p, f32)) {
+    const int rep = p.H / p.G;
+    const dim3 mg(p.B, p.G * ((rep + 31) / 32), p.num_parts);
+    switch (p.D) {
+      case 32: sink_attn_decode_mfma_kernel<1><<<mg, 64, 0, s>>>(p); break;
+      case 64: sink_attn_decode_mfma_kernel<2><<<mg, 64, 0, s>>>(p); break;
+      case 128: sink_attn_decode_mfma_kernel<4><<<mg, 64, 0, s>>>(p); break;
+      default: sink_attn_decode_mfma_kernel<8><<<mg, 64, 0, s>>>(p); break;
+    }
+  } else if (f32)
     sink_attn_decode_rows_kernel<float><<<grid, 64, sm, s>>>(p);
   else
     sink_attn_decode_rows_kernel<bf16><<<grid, 64, sm, s>>>(p);

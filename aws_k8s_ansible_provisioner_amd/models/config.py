@@ -316,6 +316,55 @@ TINY_MIXTRAL8 = register(ModelConfig(
     experts_per_token=2, bos_id=1, eos_id=2))
 
 
+def layered_config(name: str, width: int, num_layers: int, heads: int, kv_heads: int, dim: int,
+                   ff: int, chunk: int, vocab: int = 32000, loop: Optional[tuple] = None,
+                   rot_dims: Optional[int] = None, rot_base: float = 500000.0,
+                   rot_scaling: Optional[dict] = None, residual_mult: float = 1.0,
+                   embed_scale: float = 1.0, eps: float = 1e-5) -> LayeredConfig:
+    """A Bidetar-design config with `num_layers` equal layers (random-init benchmarks, tests)."""
+    spec = LayerSpec("attention",
+                     AttentionSpec(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim,
+                                   scale=dim ** -0.5,
+                                   rot=RotarySpec(rot_dims or dim, rot_base, rot_scaling),
+                                   chunk=chunk),
+                     MlpSpec("dense", ff) if ff else None)
+    cfg = LayeredConfig(name=name, hf_id="test/" + name, arch="bidetar", vocab_size=vocab,
+                        hidden_size=width, intermediate_size=ff, num_layers=0, num_heads=heads,
+                        num_kv_heads=kv_heads, head_dim=dim, rms_eps=eps, max_position=1 << 20,
+                        bos_id=0, eos_id=-1, layer_specs=[spec] * num_layers, loop=loop,
+                        embed_scale=embed_scale, residual_mult=residual_mult)
+    cfg.num_layers = len(cfg.layer_runs())
+    return cfg
+
+
+_LLAMA31_SCALING = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}
+
+# Bidetar at layer sizes of real models (random weights; bench.py --compare-design), each
+# beside a Llama-style dense model of the same width, heads, depth and feed-forward FLOPs
+# (SwiGLU's three matrices at 2/3 of the squared-ReLU feed-forward's width)
+BIDETAR_W2048 = register(layered_config(
+    "bidetar-w2048", width=2048, num_layers=16, heads=16, kv_heads=4, dim=128, ff=8192,
+    chunk=8192, rot_scaling=_LLAMA31_SCALING, residual_mult=0.5))
+LLAMA_W2048 = register(ModelConfig(
+    name="llama-w2048", hf_id="test/llama-w2048", arch="llama", vocab_size=32000,
+    hidden_size=2048, intermediate_size=5632, num_layers=16, num_heads=16, num_kv_heads=4,
+    head_dim=128, rms_eps=1e-5, rope_theta=500000.0, max_position=1 << 17, bos_id=1, eos_id=2))
+BIDETAR_W4096 = register(layered_config(
+    "bidetar-w4096", width=4096, num_layers=8, heads=32, kv_heads=8, dim=128, ff=21504,
+    chunk=8192, rot_scaling=_LLAMA31_SCALING, residual_mult=0.5))
+LLAMA_W4096 = register(ModelConfig(
+    name="llama-w4096", hf_id="test/llama-w4096", arch="llama", vocab_size=32000,
+    hidden_size=4096, intermediate_size=14336, num_layers=8, num_heads=32, num_kv_heads=8,
+    head_dim=128, rms_eps=1e-5, rope_theta=500000.0, max_position=1 << 17, bos_id=1, eos_id=2))
+# 64-wide heads, short chunks, a looped span (no D = 128-only model to set beside it)
+BIDETAR_W1536 = register(layered_config(
+    "bidetar-w1536-d64", width=1536, num_layers=8, heads=24, kv_heads=8, dim=64, ff=6144,
+    chunk=1024, loop=(2, 6, 3), rot_dims=32, residual_mult=0.5))
+TINY_BIDETAR = register(layered_config(
+    "tiny-bidetar", width=128, num_layers=3, heads=4, kv_heads=2, dim=32, ff=256, chunk=48,
+    vocab=512, loop=(1, 3, 2), rot_dims=16, residual_mult=0.7, embed_scale=4.0))
+
+
 def get_config(name: str) -> ModelConfig:
     """Resolve a registry name, HF id, or a directory holding a HF config.json."""
     if os.path.isdir(name) and os.path.exists(os.path.join(name, "config.json")):

@@ -247,8 +247,8 @@ def sink_attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
     return out
 
 
-# longest key range one decode partition covers
-DECODE_PART = 512
+# fewest keys worth a decode partition of their own
+DECODE_PART = 128
 
 
 def decode_workspace(max_seqs: int, max_heads: int, max_dim: int, max_parts: int, device):
@@ -266,7 +266,7 @@ def sink_attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Ten
                           window: int = 0, workspace=None, num_parts: int = 1) -> torch.Tensor:
     """One query per sequence, at position seq_lens[b] - 1 (seq_lens 0: a padding row, left
     unwritten); same mask, sink and gate as sink_attention_prefill.  num_parts > 1 (GPU): the
-    visible key range is cut into num_parts partitions of whole DECODE_PART-key pieces, one
+    visible key range is cut into num_parts equal partitions (whole 32- or 64-key pieces), one
     workgroup each, merged by a second launch (workspace from decode_workspace)."""
     if _native(q):
         ws_ml, ws_o = workspace if (workspace is not None and num_parts > 1) else (None, None)

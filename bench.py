@@ -89,7 +89,85 @@ def parse():
                          "kernel table")
     ap.add_argument("--profile-steps", type=int, default=0,
                     help="extra untimed waves run after timing (for rocprofv3 captures)")
+    ap.add_argument("--compare-design", default=None, choices=["bidetar"],
+                    help="instead of the serving wave: prefill and decode throughput of this "
+                         "design at real layer sizes (random weights) beside the closest "
+                         "existing model of equal size; prints one JSON line with the table")
+    ap.add_argument("--compare-models", default=None,
+                    help="comma list of registry names for --compare-design (default: the "
+                         "design's registered sizes and their dense counterparts)")
     return ap.parse_args()
+
+
+COMPARE_SETS = {
+    # (model of the design, closest existing model of equal size or None)
+    "bidetar": [("bidetar-w2048", "llama-w2048"), ("bidetar-w4096", "llama-w4096"),
+                ("bidetar-w1536-d64", None)],
+}
+
+
+def compare_design(a) -> int:
+    """Prefill and decode throughput per model through the engine (random weights, one GPU):
+    prefill = `P` prompts of `L` tokens served to their first token (chunked prefill steps of
+    max_num_batched_tokens); decode = `B` sequences of context ~L generating `O` tokens
+    (hipGraph decode), timed as the difference between a run to 1 token and a run to O + 1."""
+    import torch
+
+    from aws_k8s_ansible_provisioner_amd.engine.config import EngineConfig, SamplingParams
+    from aws_k8s_ansible_provisioner_amd.engine.llm_engine import LLMEngine
+    from aws_k8s_ansible_provisioner_amd.models.config import get_config
+
+    if a.compare_models:
+        pairs = [(m, None) for m in a.compare_models.split(",")]
+    else:
+        pairs = COMPARE_SETS[a.compare_design]
+    P, L, B, O = 16, a.input_len * 4, 64, a.output_len // 2
+    dev = a.device
+    gpu = dev != "cpu" and torch.cuda.is_available()
+    if not gpu:
+        P, L, B, O = 2, 64, 2, 4
+    rows = []
+    rng = np.random.default_rng(0)
+
+    def run(eng, n, plen, out_len):
+        prompts = [rng.integers(3, eng.mcfg.vocab_size, plen).tolist() for _ in range(n)]
+        if gpu:
+            torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.generate(None, SamplingParams(max_tokens=out_len, temperature=0.0, ignore_eos=True),
+                     prompt_ids=prompts)
+        if gpu:
+            torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    for pair in pairs:
+        for name in pair:
+            if name is None:
+                continue
+            mcfg = get_config(name)
+            blocks = (max(P, B) * (L + O + 64)) // a.block_size + 64
+            eng = LLMEngine(EngineConfig(
+                model=name, max_model_len=L + O + 64, max_num_seqs=B, cuda_graph_max_bs=B,
+                max_num_batched_tokens=a.max_num_batched_tokens, block_size=a.block_size,
+                num_gpu_blocks=blocks, enable_prefix_caching=False, device=dev,
+                enforce_eager=a.enforce_eager, init_std=0.02),
+                log=lambda *x: print(*x, file=sys.stderr, flush=True))
+            run(eng, 2, min(L, 256), 2)  # warm-up
+            tp = min(run(eng, P, L, 1) for _ in range(max(1, a.steps)))
+            t1 = min(run(eng, B, L, 1) for _ in range(max(1, a.steps)))
+            t2 = min(run(eng, B, L, O + 1) for _ in range(max(1, a.steps)))
+            rows.append({"model": name, "design": mcfg.arch,
+                         "params_b": round(mcfg.num_params() / 1e9, 3),
+                         "prefill_tok_s": round(P * L / tp, 1),
+                         "decode_tok_s": round(B * O / max(t2 - t1, 1e-9), 1),
+                         "prefill": f"{P}x{L}", "decode": f"{B} seqs, ctx {L}..{L + O}"})
+            print(f"[compare] {rows[-1]}", file=sys.stderr, flush=True)
+            del eng
+            if gpu:
+                torch.cuda.empty_cache()
+    print(json.dumps({"compare_design": a.compare_design, "dtype": "bf16", "data": "synthetic",
+                      "rows": rows}), flush=True)
+    return 0
 
 
 def physical_devices(devs: list) -> int:
@@ -133,6 +211,8 @@ def self_launch(a) -> int | None:
 
 def main() -> int:
     a = parse()
+    if a.compare_design:
+        return compare_design(a)
     rc = self_launch(a)
     if rc is not None:
         return rc

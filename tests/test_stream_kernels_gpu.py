@@ -95,6 +95,7 @@ CASES = [  # H, G, D, chunk, window, sink, gate
     (2, 2, 80, 64, 33, True, True),
     (3, 1, 256, 1000, 0, False, False),
     (16, 2, 128, 512, 0, True, True),
+    (40, 1, 32, 90, 0, True, True),     # more query heads per K/V head than one 32-column tile
 ]
 
 
