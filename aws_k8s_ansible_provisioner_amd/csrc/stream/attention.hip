@@ -23,6 +23,8 @@
 //   from accumulator to B operand without any lane movement, and the V^T operand is one
 //   16-byte load from the grouped V cache.  K / V fragments come straight from global memory
 //   (L1 / L2 hits across the workgroup's four waves and the heads of a GQA group).
+#include <cstdlib>
+
 #include "../kernels/common.h"
 #include "stream.h"
 
@@ -309,61 +311,100 @@ struct MfmaState {
 
 // Keys [jb, je] (jb a multiple of 32) against the wave's query columns.  qf: the columns' Q
 // fragments (B operands); pos / my_lo: each lane's query position and lowest visible key per
-// tile (my_lo > pos: an unused column).  Each K and V fragment is loaded once, straight from
-// the cache, and feeds the MFMAs of all NQ tiles.
+// tile; pos_min / lo_max: the smallest position and the largest lower bound among the wave's
+// columns (an unused column computes like a used one and is never stored).  m is kept in log2
+// units of the scaled scores.  Each K and V fragment is loaded once, straight from the cache,
+// and feeds the MFMAs of all NQ tiles.
 template <int DB, int NQ>
 __device__ __forceinline__ void mfma_attend(MfmaState<DB, NQ>& st, const AttnParams& p,
                                             const int32_t* __restrict__ bt, int g,
                                             const akap::bf16x8 (&qf)[NQ][2 * DB],
                                             const int (&pos)[NQ], const int (&my_lo)[NQ], int jb,
-                                            int je) {
+                                            int je, int pos_min, int lo_max) {
   constexpr int D = 32 * DB, KS = 2 * DB;
+  const float sc2 = p.scale * 1.44269504088896f;  // scores -> log2 units
   using akap::bf16x8;
   using akap::f32x16;
   const int lane = threadIdx.x & 63;
   const int col = lane & 31, hf = lane >> 5;
   const int NG = p.BS >> 3;
   const int krow = swap23(col);
-  for (int j0 = jb; j0 <= je; j0 += 32) {
+  // The next block's K fragments are requested before this block's softmax, and this block's
+  // V fragments before its Q K^T MFMAs: a wave keeps its own loads in flight under its own
+  // matrix and VALU work (the accumulators leave room for one or two waves per SIMD only).
+  auto block_of = [&](int j0) {
     const int bi = j0 / p.BS;
     int blk = bi < p.max_blocks ? bt[bi] : 0;
     if (blk < 0 || blk >= p.NB) blk = 0;
-    const int off0 = j0 - bi * p.BS;  // a multiple of 32: the 32 keys lie in one block
-    const bf16* kp = (const bf16*)p.k_cache +
-                     ((size_t)(blk * p.G + g) * p.BS + off0 + krow) * D + 8 * hf;
-    const bf16* vp = (const bf16*)p.v_cache +
-                     (((size_t)(blk * p.G + g) * NG + (off0 >> 3) + hf) * D + col) * 8;
-    bf16x8 kf[KS];
+    return (blk * p.G + g) * p.BS + (j0 - bi * p.BS);  // row of key j0 in the [.., D] K view
+  };
+  bf16x8 kf[KS];
+  int row0 = block_of(jb);
+  {
+    const bf16* kp = (const bf16*)p.k_cache + ((size_t)row0 + krow) * D + 8 * hf;
 #pragma unroll
     for (int c = 0; c < KS; ++c) kf[c] = *reinterpret_cast<const bf16x8*>(kp + 16 * c);
-    bf16x8 pb[NQ][2];
-    float alpha[NQ];
+  }
+  for (int j0 = jb; j0 <= je; j0 += 32) {
+    // V groups of this block: row0 is a multiple of 8 keys (blocks and j0 are multiples of 32)
+    const bf16* vp = (const bf16*)p.v_cache + (((size_t)(row0 >> 3) + hf) * D + col) * 8;
+    bf16x8 vf[DB][2];
+#pragma unroll
+    for (int dt = 0; dt < DB; ++dt)
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl)
+        vf[dt][sl] = *reinterpret_cast<const bf16x8*>(vp + ((size_t)(2 * sl) * D + 32 * dt) * 8);
+    f32x16 s[NQ];
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
-      f32x16 s;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[i] = 0.f;
+      for (int i = 0; i < 16; ++i) s[q][i] = 0.f;
 #pragma unroll
       for (int c = 0; c < KS; ++c)
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[c], qf[q][c], s, 0, 0, 0);
+        s[q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[c], qf[q][c], s[q], 0, 0, 0);
+    }
+    if (j0 + 32 <= je) {
+      row0 = block_of(j0 + 32);
+      const bf16* kp = (const bf16*)p.k_cache + ((size_t)row0 + krow) * D + 8 * hf;
+#pragma unroll
+      for (int c = 0; c < KS; ++c) kf[c] = *reinterpret_cast<const bf16x8*>(kp + 16 * c);
+    }
+    bf16x8 pb[NQ][2];
+    float alpha[NQ];
+    // a block below every column's position and above every column's lower bound needs no
+    // mask (all but the first and last blocks of a wave's range)
+    const bool full = j0 + 31 <= pos_min && j0 >= lo_max;
+    bool rescale = false;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
       // accumulator register i of this lane: key j0 + 16 (i >> 3) + 8 hf + (i & 7), column col
       float sv[16];
       float bmax = -INFINITY;
+      if (full) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = j0 + 16 * (i >> 3) + 8 * hf + (i & 7);
-        const bool vis = key <= pos[q] && key >= my_lo[q];
-        sv[i] = vis ? s[i] * p.scale : -INFINITY;
-        bmax = fmaxf(bmax, sv[i]);
+        for (int i = 0; i < 16; ++i) {
+          sv[i] = s[q][i];
+          bmax = fmaxf(bmax, sv[i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = j0 + 16 * (i >> 3) + 8 * hf + (i & 7);
+          const bool vis = key <= pos[q] && key >= my_lo[q];
+          sv[i] = vis ? s[q][i] : -INFINITY;
+          bmax = fmaxf(bmax, sv[i]);
+        }
       }
       bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
-      const float mn = fmaxf(st.m[q], bmax);
+      // running max and exponentials in the log2 domain of the scaled scores (sc2 > 0)
+      const float mn = fmaxf(st.m[q], bmax * sc2);
       const float ms = mn == -INFINITY ? 0.f : mn;  // nothing visible yet: every exp below is 0
-      alpha[q] = __expf(st.m[q] - ms);
+      alpha[q] = __builtin_amdgcn_exp2f(st.m[q] - ms);
+      rescale |= alpha[q] != 1.0f;
       float psum = 0.f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        sv[i] = __expf(sv[i] - ms);
+        sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -ms));
         psum += sv[i];
       }
       psum += __shfl_xor(psum, 32, 64);
@@ -372,21 +413,22 @@ __device__ __forceinline__ void mfma_attend(MfmaState<DB, NQ>& st, const AttnPar
 #pragma unroll
       for (int i = 0; i < 16; ++i) pb[q][i >> 3][i & 7] = (bf16)sv[i];
     }
+    if (__any(rescale)) {  // (wave-uniform) the maxima settle after the first blocks
 #pragma unroll
-    for (int dt = 0; dt < DB; ++dt) {
-#pragma unroll
-      for (int q = 0; q < NQ; ++q)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) st.o[q][dt][i] *= alpha[q];
-#pragma unroll
-      for (int sl = 0; sl < 2; ++sl) {
-        const bf16x8 vf =
-            *reinterpret_cast<const bf16x8*>(vp + ((size_t)(2 * sl) * D + 32 * dt) * 8);
+      for (int dt = 0; dt < DB; ++dt)
 #pragma unroll
         for (int q = 0; q < NQ; ++q)
-          st.o[q][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[q][sl], st.o[q][dt], 0, 0, 0);
-      }
+#pragma unroll
+          for (int i = 0; i < 16; ++i) st.o[q][dt][i] *= alpha[q];
     }
+#pragma unroll
+    for (int dt = 0; dt < DB; ++dt)
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl)
+#pragma unroll
+        for (int q = 0; q < NQ; ++q)
+          st.o[q][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][sl], pb[q][sl], st.o[q][dt],
+                                                                0, 0, 0);
   }
 }
 
@@ -413,8 +455,9 @@ __device__ __forceinline__ void mfma_finish(const MfmaState<DB, NQ>& st, int q,
   float l = st.l[q], corr = 1.f;
   if (p.sink) {
     const float sk = p.sink[h];
-    const float mf = fmaxf(st.m[q], sk);
-    corr = expf(st.m[q] - mf);
+    const float mq = st.m[q] * 0.693147180559945f;  // back from log2 units
+    const float mf = fmaxf(mq, sk);
+    corr = expf(mq - mf);
     l = l * corr + expf(sk - mf);
   }
   float gate = 1.f;
@@ -431,10 +474,10 @@ __device__ __forceinline__ void mfma_finish(const MfmaState<DB, NQ>& st, int q,
       o[32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = (bf16)(st.o[q][dt][i] * f);
 }
 
-// Prefill: grid (tiles of 128 tokens, H), 2 waves of 64 queries (two column tiles) each.
-template <int DB>
-__global__ __launch_bounds__(128) void sink_attn_prefill_mfma_kernel(AttnParams p) {
-  constexpr int D = 32 * DB, KS = 2 * DB, NQ = 2;
+// Prefill: grid (tiles of 128 tokens, H), 128 / (32 NQ) waves of NQ column tiles each.
+template <int DB, int NQ>
+__global__ __launch_bounds__(128 / NQ * 2) void sink_attn_prefill_mfma_kernel(AttnParams p) {
+  constexpr int D = 32 * DB, KS = 2 * DB;
   using akap::bf16x8;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int col = lane & 31, hf = lane >> 5;
@@ -445,7 +488,7 @@ __global__ __launch_bounds__(128) void sink_attn_prefill_mfma_kernel(AttnParams 
   const int qlen = p.q_start[b + 1] - qs0;
   const int kv = p.seq_lens[b];
   const int rend = min(p.tile_row[tile] + p.tile_rows, qlen);
-  const int r0 = p.tile_row[tile] + wave * 64;
+  const int r0 = p.tile_row[tile] + wave * 32 * NQ;
   if (r0 >= rend || kv < qlen) return;
   const int g = h / (p.H / p.G);
   const int32_t* bt = p.block_tables + (size_t)b * p.max_blocks;
@@ -458,16 +501,21 @@ __global__ __launch_bounds__(128) void sink_attn_prefill_mfma_kernel(AttnParams 
     valid[q] = r < rend;
     t[q] = qs0 + (valid[q] ? r : r0);
     pos[q] = kv - qlen + r;
-    my_lo[q] = valid[q] ? lower_bound_of(pos[q], p.chunk, p.window) : 0x7fffffff;
+    my_lo[q] = lower_bound_of(pos[q], p.chunk, p.window);
     const bf16* qp = (const bf16*)p.q + ((size_t)t[q] * p.H + h) * D + 8 * hf;
 #pragma unroll
     for (int c = 0; c < KS; ++c) qf[q][c] = *reinterpret_cast<const bf16x8*>(qp + 16 * c);
   }
-  const int pos_last = kv - qlen + min(r0 + 63, rend - 1);
+  const int pos_last = kv - qlen + min(r0 + 32 * NQ - 1, rend - 1);
   const int lo_w = lower_bound_of(kv - qlen + r0, p.chunk, p.window);
   MfmaState<DB, NQ> st;
   mfma_init(st);
-  mfma_attend<DB, NQ>(st, p, bt, g, qf, pos, my_lo, lo_w & ~31, pos_last);
+  // columns past the tile's end compute like real ones (positions past the last key are
+  // masked by the range, never read) and are not stored
+  const int pos_first = kv - qlen + r0;
+  const int lo_max = lower_bound_of(kv - qlen + r0 + 32 * NQ - 1, p.chunk, p.window);
+  mfma_attend<DB, NQ>(st, p, bt, g, qf, pos, my_lo, lo_w & ~31, pos_last, pos_first,
+                      max(lo_w, lo_max));
 #pragma unroll
   for (int q = 0; q < NQ; ++q)
     if (valid[q]) mfma_finish<DB, NQ>(st, q, p, t[q], h);
@@ -502,7 +550,7 @@ __global__ __launch_bounds__(64) void sink_attn_decode_mfma_kernel(AttnParams p)
   per = (per + 31) & ~31;
   const int jb = a0 + part * per;
   const int je = min(pos1, jb + per - 1);
-  int pos[1] = {pos1}, my_lo[1] = {valid ? lo : 0x7fffffff};
+  int pos[1] = {pos1}, my_lo[1] = {lo};
   bf16x8 qf[1][KS];
   {
     const bf16* qp = (const bf16*)p.q + ((size_t)b * p.H + h) * D + 8 * hf;
@@ -512,7 +560,8 @@ __global__ __launch_bounds__(64) void sink_attn_decode_mfma_kernel(AttnParams p)
   MfmaState<DB, 1> st;
   mfma_init(st);
   if (jb <= je)
-    mfma_attend<DB, 1>(st, p, p.block_tables + (size_t)b * p.max_blocks, g, qf, pos, my_lo, jb, je);
+    mfma_attend<DB, 1>(st, p, p.block_tables + (size_t)b * p.max_blocks, g, qf, pos, my_lo, jb, je,
+                       pos1, lo);
   if (!valid) return;
   if (p.num_parts == 1) {
     mfma_finish<DB, 1>(st, 0, p, b, h);
@@ -520,7 +569,7 @@ __global__ __launch_bounds__(64) void sink_attn_decode_mfma_kernel(AttnParams p)
   }
   const size_t slot = ((size_t)b * p.H + h) * p.num_parts + part;
   if (hf == 0) {
-    p.ws_ml[slot * 2] = st.m[0];
+    p.ws_ml[slot * 2] = st.m[0] * 0.693147180559945f;  // the merge works in natural units
     p.ws_ml[slot * 2 + 1] = st.l[0];
   }
 #pragma unroll
@@ -532,18 +581,31 @@ __global__ __launch_bounds__(64) void sink_attn_decode_mfma_kernel(AttnParams p)
 
 // the matrix kernels take bf16 and these head sizes (prefill: tiles of 128 tokens)
 static bool mfma_ok(const AttnParams& p, bool f32) {
-  return !f32 && (p.D == 32 || p.D == 64 || p.D == 128 || p.D == 256) && p.BS % 32 == 0;
+  return !f32 && (p.D == 32 || p.D == 64 || p.D == 128 || p.D == 256) && p.BS % 32 == 0 &&
+         p.scale > 0.f;  // (the running max is taken on unscaled scores)
 }
 
 void launch_sink_attention_prefill(const AttnParams& p, bool f32, hipStream_t s) {
   if (p.num_tiles <= 0) return;
   const dim3 grid(p.num_tiles, p.H);
   if (mfma_ok(p, f32) && p.tile_rows == 128) {
-    switch (p.D) {
-      case 32: sink_attn_prefill_mfma_kernel<1><<<grid, 128, 0, s>>>(p); break;
-      case 64: sink_attn_prefill_mfma_kernel<2><<<grid, 128, 0, s>>>(p); break;
-      case 128: sink_attn_prefill_mfma_kernel<4><<<grid, 128, 0, s>>>(p); break;
-      default: sink_attn_prefill_mfma_kernel<8><<<grid, 128, 0, s>>>(p); break;
+    static const int nq = [] {  // AKAP_STREAM_NQ=1|2: column tiles per wave (A/B knob)
+      const char* e = getenv("AKAP_STREAM_NQ");
+      return e ? atoi(e) : 2;
+    }();
+    if (nq == 1 || p.D == 256) {
+      switch (p.D) {
+        case 32: sink_attn_prefill_mfma_kernel<1, 1><<<grid, 256, 0, s>>>(p); break;
+        case 64: sink_attn_prefill_mfma_kernel<2, 1><<<grid, 256, 0, s>>>(p); break;
+        case 128: sink_attn_prefill_mfma_kernel<4, 1><<<grid, 256, 0, s>>>(p); break;
+        default: sink_attn_prefill_mfma_kernel<8, 1><<<grid, 256, 0, s>>>(p); break;
+      }
+    } else {
+      switch (p.D) {
+        case 32: sink_attn_prefill_mfma_kernel<1, 2><<<grid, 128, 0, s>>>(p); break;
+        case 64: sink_attn_prefill_mfma_kernel<2, 2><<<grid, 128, 0, s>>>(p); break;
+        default: sink_attn_prefill_mfma_kernel<4, 2><<<grid, 128, 0, s>>>(p); break;
+      }
     }
     return;
   }
