@@ -309,6 +309,68 @@ struct MfmaState {
   float m[NQ], l[NQ];
 };
 
+// Softmax update of one 32-key block: masks (unless the block is visible to every column),
+// moves the running max and sum (log2 domain), turns the scores of the NQ tiles into bf16 P
+// operands and rescales the output accumulators if a maximum moved.
+template <int DB, int NQ>
+__device__ __forceinline__ void mfma_softmax(MfmaState<DB, NQ>& st, akap::f32x16 (&s)[NQ],
+                                             akap::bf16x8 (&pb)[NQ][2], int j0,
+                                             const int (&pos)[NQ], const int (&my_lo)[NQ],
+                                             int pos_min, int lo_max, float sc2) {
+  const int hf = (threadIdx.x & 63) >> 5;
+  float alpha[NQ];
+  // a block below every column's position and above every column's lower bound needs no
+  // mask (all but the first and last blocks of a wave's range)
+  const bool full = j0 + 31 <= pos_min && j0 >= lo_max;
+  bool rescale = false;
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    // accumulator register i of this lane: key j0 + 16 (i >> 3) + 8 hf + (i & 7), column col
+    float sv[16];
+    float bmax = -INFINITY;
+    if (full) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        sv[i] = s[q][i];
+        bmax = fmaxf(bmax, sv[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = j0 + 16 * (i >> 3) + 8 * hf + (i & 7);
+        const bool vis = key <= pos[q] && key >= my_lo[q];
+        sv[i] = vis ? s[q][i] : -INFINITY;
+        bmax = fmaxf(bmax, sv[i]);
+      }
+    }
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    // running max and exponentials in the log2 domain of the scaled scores (sc2 > 0)
+    const float mn = fmaxf(st.m[q], bmax * sc2);
+    const float ms = mn == -INFINITY ? 0.f : mn;  // nothing visible yet: every exp below is 0
+    alpha[q] = __builtin_amdgcn_exp2f(st.m[q] - ms);
+    rescale |= alpha[q] != 1.0f;
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -ms));
+      psum += sv[i];
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    st.l[q] = st.l[q] * alpha[q] + psum;
+    st.m[q] = mn;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) pb[q][i >> 3][i & 7] = (bf16)sv[i];
+  }
+  if (__any(rescale)) {  // (wave-uniform) the maxima settle after the first blocks
+#pragma unroll
+    for (int dt = 0; dt < DB; ++dt)
+#pragma unroll
+      for (int q = 0; q < NQ; ++q)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) st.o[q][dt][i] *= alpha[q];
+  }
+}
+
 // Keys [jb, je] (jb a multiple of 32) against the wave's query columns.  qf: the columns' Q
 // fragments (B operands); pos / my_lo: each lane's query position and lowest visible key per
 // tile; pos_min / lo_max: the smallest position and the largest lower bound among the wave's
@@ -340,6 +402,12 @@ __device__ __forceinline__ void mfma_attend(MfmaState<DB, NQ>& st, const AttnPar
   };
   bf16x8 kf[KS];
   int row0 = block_of(jb);
+  // one column tile per wave: the block-table entry of the block after next is requested a
+  // whole iteration before the K loads that need it (no K load waits on a table load; 715 ->
+  // 591 us at 8 x 2048 causal, D = 128).  With two tiles the extra live state costs the last
+  // free registers (534 -> 697 us), so there the entry is looked up when it is needed.
+  constexpr bool kTableAhead = NQ == 1;
+  int row1 = kTableAhead && jb + 32 <= je ? block_of(jb + 32) : 0;
   {
     const bf16* kp = (const bf16*)p.k_cache + ((size_t)row0 + krow) * D + 8 * hf;
 #pragma unroll
@@ -364,63 +432,14 @@ __device__ __forceinline__ void mfma_attend(MfmaState<DB, NQ>& st, const AttnPar
         s[q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[c], qf[q][c], s[q], 0, 0, 0);
     }
     if (j0 + 32 <= je) {
-      row0 = block_of(j0 + 32);
+      row0 = kTableAhead ? row1 : block_of(j0 + 32);
       const bf16* kp = (const bf16*)p.k_cache + ((size_t)row0 + krow) * D + 8 * hf;
 #pragma unroll
       for (int c = 0; c < KS; ++c) kf[c] = *reinterpret_cast<const bf16x8*>(kp + 16 * c);
+      if (kTableAhead && j0 + 64 <= je) row1 = block_of(j0 + 64);
     }
     bf16x8 pb[NQ][2];
-    float alpha[NQ];
-    // a block below every column's position and above every column's lower bound needs no
-    // mask (all but the first and last blocks of a wave's range)
-    const bool full = j0 + 31 <= pos_min && j0 >= lo_max;
-    bool rescale = false;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      // accumulator register i of this lane: key j0 + 16 (i >> 3) + 8 hf + (i & 7), column col
-      float sv[16];
-      float bmax = -INFINITY;
-      if (full) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          sv[i] = s[q][i];
-          bmax = fmaxf(bmax, sv[i]);
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = j0 + 16 * (i >> 3) + 8 * hf + (i & 7);
-          const bool vis = key <= pos[q] && key >= my_lo[q];
-          sv[i] = vis ? s[q][i] : -INFINITY;
-          bmax = fmaxf(bmax, sv[i]);
-        }
-      }
-      bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
-      // running max and exponentials in the log2 domain of the scaled scores (sc2 > 0)
-      const float mn = fmaxf(st.m[q], bmax * sc2);
-      const float ms = mn == -INFINITY ? 0.f : mn;  // nothing visible yet: every exp below is 0
-      alpha[q] = __builtin_amdgcn_exp2f(st.m[q] - ms);
-      rescale |= alpha[q] != 1.0f;
-      float psum = 0.f;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -ms));
-        psum += sv[i];
-      }
-      psum += __shfl_xor(psum, 32, 64);
-      st.l[q] = st.l[q] * alpha[q] + psum;
-      st.m[q] = mn;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) pb[q][i >> 3][i & 7] = (bf16)sv[i];
-    }
-    if (__any(rescale)) {  // (wave-uniform) the maxima settle after the first blocks
-#pragma unroll
-      for (int dt = 0; dt < DB; ++dt)
-#pragma unroll
-        for (int q = 0; q < NQ; ++q)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) st.o[q][dt][i] *= alpha[q];
-    }
+    mfma_softmax<DB, NQ>(st, s, pb, j0, pos, my_lo, pos_min, lo_max, sc2);
 #pragma unroll
     for (int dt = 0; dt < DB; ++dt)
 #pragma unroll
@@ -474,9 +493,9 @@ __device__ __forceinline__ void mfma_finish(const MfmaState<DB, NQ>& st, int q,
       o[32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = (bf16)(st.o[q][dt][i] * f);
 }
 
-// Prefill: grid (tiles of 128 tokens, H), 128 / (32 NQ) waves of NQ column tiles each.
+// Prefill: grid (tiles of 128 or 256 tokens, H), tile / (32 NQ) waves of NQ column tiles each.
 template <int DB, int NQ>
-__global__ __launch_bounds__(128 / NQ * 2) void sink_attn_prefill_mfma_kernel(AttnParams p) {
+__global__ __launch_bounds__(512 / NQ) void sink_attn_prefill_mfma_kernel(AttnParams p) {
   constexpr int D = 32 * DB, KS = 2 * DB;
   using akap::bf16x8;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -588,23 +607,24 @@ static bool mfma_ok(const AttnParams& p, bool f32) {
 void launch_sink_attention_prefill(const AttnParams& p, bool f32, hipStream_t s) {
   if (p.num_tiles <= 0) return;
   const dim3 grid(p.num_tiles, p.H);
-  if (mfma_ok(p, f32) && p.tile_rows == 128) {
+  if (mfma_ok(p, f32) && (p.tile_rows == 128 || p.tile_rows == 256)) {
+    const int tr = p.tile_rows;
     static const int nq = [] {  // AKAP_STREAM_NQ=1|2: column tiles per wave (A/B knob)
       const char* e = getenv("AKAP_STREAM_NQ");
       return e ? atoi(e) : 2;
     }();
     if (nq == 1 || p.D == 256) {
       switch (p.D) {
-        case 32: sink_attn_prefill_mfma_kernel<1, 1><<<grid, 256, 0, s>>>(p); break;
-        case 64: sink_attn_prefill_mfma_kernel<2, 1><<<grid, 256, 0, s>>>(p); break;
-        case 128: sink_attn_prefill_mfma_kernel<4, 1><<<grid, 256, 0, s>>>(p); break;
-        default: sink_attn_prefill_mfma_kernel<8, 1><<<grid, 256, 0, s>>>(p); break;
+        case 32: sink_attn_prefill_mfma_kernel<1, 1><<<grid, 2 * tr, 0, s>>>(p); break;
+        case 64: sink_attn_prefill_mfma_kernel<2, 1><<<grid, 2 * tr, 0, s>>>(p); break;
+        case 128: sink_attn_prefill_mfma_kernel<4, 1><<<grid, 2 * tr, 0, s>>>(p); break;
+        default: sink_attn_prefill_mfma_kernel<8, 1><<<grid, 2 * tr, 0, s>>>(p); break;
       }
     } else {
       switch (p.D) {
-        case 32: sink_attn_prefill_mfma_kernel<1, 2><<<grid, 128, 0, s>>>(p); break;
-        case 64: sink_attn_prefill_mfma_kernel<2, 2><<<grid, 128, 0, s>>>(p); break;
-        default: sink_attn_prefill_mfma_kernel<4, 2><<<grid, 128, 0, s>>>(p); break;
+        case 32: sink_attn_prefill_mfma_kernel<1, 2><<<grid, tr, 0, s>>>(p); break;
+        case 64: sink_attn_prefill_mfma_kernel<2, 2><<<grid, tr, 0, s>>>(p); break;
+        default: sink_attn_prefill_mfma_kernel<4, 2><<<grid, tr, 0, s>>>(p); break;
       }
     }
     return;

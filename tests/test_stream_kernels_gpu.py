@@ -100,7 +100,7 @@ CASES = [  # H, G, D, chunk, window, sink, gate
 
 
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("tr", [64, 128])   # 128-token tiles in bf16: the matrix-core kernel
+@pytest.mark.parametrize("tr", [64, 128, 256])   # 128 / 256-token tiles in bf16: matrix cores
 @pytest.mark.parametrize("H,G,D,chunk,window,use_sink,use_gate", CASES)
 def test_sink_attention_prefill(dt, tr, H, G, D, chunk, window, use_sink, use_gate):
     g = torch.Generator().manual_seed(H + D + chunk + window)
