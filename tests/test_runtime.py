@@ -521,3 +521,45 @@ def test_prefill_tile_map_sorted_by_causal_work_with_context():
         work.append(sl[seqs[t]] - q + min(q, -(-(rows[t] + 64) // 2)))
     assert work == sorted(work) and work == [3, 60]  # fresh 3-token tile, then 40 + 20 keys
     assert sorted(zip(seqs, rows)) == sorted(set(zip(seqs, rows)))  # no tile lost or doubled
+
+
+def test_forced_steps_lay_out_single_tokens_first_and_reuse_pages():
+    """schedule_forced: the caller dictates each request's tokens.  Single-token entries lead
+    the batch as decode rows, chunks follow in the caller's order; positions and slots continue
+    from what earlier steps left; ended requests give their pages back."""
+    s, b = _sched(num_blocks=6, bs=4, max_seqs=3, budget=32, max_len=16, prefix=False, G=1)
+    i = s.schedule_forced([(7, [10, 11, 12, 13, 14]), (8, [20]), (9, [30, 31])], b)
+    assert i["is_prefill"] and i["num_decode"] == 1 and i["num_seqs"] == 3 and i["num_tokens"] == 8
+    assert i["num_samples"] == 0 and list(i["entry_row"]) == [1, 0, 6]
+    assert list(b["req_ids"][:3]) == [8, 7, 9] and list(b["q_start"][:4]) == [0, 1, 6, 8]
+    assert list(b["input_ids"][:8]) == [20, 10, 11, 12, 13, 14, 30, 31]
+    assert list(b["positions"][:8]) == [0, 0, 1, 2, 3, 4, 0, 1]
+    assert list(b["seq_lens"][:3]) == [1, 5, 2] and i["num_tiles"] == 2
+    assert s.num_running == 3 and s.num_free_blocks() == 2
+    # request 9 is left out of a step and goes on later; 7 and 8 decode alone: a pure decode step
+    i = s.schedule_forced([(7, [15]), (8, [21])], b)
+    assert not i["is_prefill"] and i["num_decode"] == 2 and i["num_samples"] == 2
+    assert list(b["positions"][:2]) == [5, 1] and list(b["seq_lens"][:2]) == [6, 2]
+    bt = b["block_tables"].reshape(3, 4)
+    assert list(b["slots"][:2]) == [bt[0][1] * 4 + 1, bt[1][0] * 4 + 1]
+    for rid in (7, 8):
+        assert s.abort_request(rid)
+        s.release(rid)
+    assert s.num_free_blocks() == 5 and s.num_running == 1
+    i = s.schedule_forced([(9, [32, 33, 34]), (11, list(range(40, 52)))], b)   # pages used again
+    assert list(b["positions"][:3]) == [2, 3, 4] and list(i["entry_row"]) == [0, 3]
+    assert s.num_free_blocks() == 1
+
+
+def test_forced_steps_refuse_what_does_not_fit_and_change_nothing():
+    s, b = _sched(num_blocks=3, bs=4, max_seqs=2, budget=32, max_len=16, prefix=False, G=1)
+    s.schedule_forced([(1, [5, 6, 7])], b)
+    for bad in ([(1, [8]), (1, [9])],                 # twice in one step
+                [(1, [])],                            # no tokens
+                [(1, [8]), (2, [1]), (3, [1])],       # more entries than sequence slots
+                [(1, list(range(14)))]):              # longer than the model length
+        with pytest.raises(ValueError):
+            s.schedule_forced(bad, b)
+    assert s.num_running == 1 and s.request_info(1)["num_tokens"] == 3
+    with pytest.raises(RuntimeError):                 # 3 pages cannot hold 3 + 11 tokens
+        s.schedule_forced([(1, [8]), (2, list(range(11)))], b)
