@@ -914,8 +914,35 @@ struct CarComm {
   akap::CarArgs args{};
   void* buf = nullptr;
   void* sig = nullptr;
+  size_t buf_bytes = 0, sig_bytes = 0;
   std::vector<void*> opened;
 };
+// Uncached (MTYPE UC) allocations are never returned to the driver before the process ends:
+// after a hipFree of uncached memory that a kernel has read, tensors allocated later in the
+// same address range have held wrong values.  A destroyed communicator parks its buffers here
+// and the next one of the same device and size takes them over.
+struct UncachedBlock {
+  int device;
+  size_t bytes;
+  void* ptr;
+};
+std::vector<UncachedBlock>& uncached_pool() {
+  static std::vector<UncachedBlock> p;
+  return p;
+}
+hipError_t uncached_alloc(void** out, size_t bytes, int device) {
+  auto& pool = uncached_pool();
+  for (size_t i = 0; i < pool.size(); ++i)
+    if (pool[i].device == device && pool[i].bytes == bytes) {
+      *out = pool[i].ptr;
+      pool.erase(pool.begin() + i);
+      return hipSuccess;
+    }
+  return hipExtMallocWithFlags(out, bytes, hipDeviceMallocUncached);
+}
+void uncached_release(void* ptr, size_t bytes, int device) {
+  if (ptr != nullptr) uncached_pool().push_back({device, bytes, ptr});
+}
 std::vector<CarComm*>& car_table() {
   static std::vector<CarComm*> t;
   return t;
@@ -942,8 +969,10 @@ int64_t car_create(int64_t device, int64_t rank, int64_t world, int64_t max_elem
   c->device = (int)device;
   const size_t buf_bytes = (size_t)4 * max_elems * sizeof(uint16_t);
   const size_t sig_bytes = akap::custom_allreduce_signal_bytes();
-  HIP_OK(hipExtMallocWithFlags(&c->buf, buf_bytes, hipDeviceMallocUncached));
-  HIP_OK(hipExtMallocWithFlags(&c->sig, sig_bytes, hipDeviceMallocUncached));
+  HIP_OK(uncached_alloc(&c->buf, buf_bytes, (int)device));
+  HIP_OK(uncached_alloc(&c->sig, sig_bytes, (int)device));
+  c->buf_bytes = buf_bytes;
+  c->sig_bytes = sig_bytes;
   HIP_OK(hipMemset(c->sig, 0, sig_bytes));
   void* local = nullptr;
   HIP_OK(hipMalloc(&local, 4096));
@@ -1238,8 +1267,8 @@ void car_destroy(int64_t h) {
   const c10::DeviceGuard g(c10::Device(c10::DeviceType::CUDA, c->device));
   (void)hipDeviceSynchronize();
   for (void* p : c->opened) (void)hipIpcCloseMemHandle(p);
-  (void)hipFree(c->buf);
-  (void)hipFree(c->sig);
+  uncached_release(c->buf, c->buf_bytes, c->device);
+  uncached_release(c->sig, c->sig_bytes, c->device);
   (void)hipFree(c->args.counter);
   delete c;
   car_table()[h] = nullptr;
