@@ -63,7 +63,7 @@ def test_small_pool_is_used_again(model, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decode_through_graphs_and_split_partitions(tmp_path, dtype):
-    """Decode far past the 512-key partition length of the split decode kernel, over a full-
+    """Decode over a key range that the split decode kernel cuts into several partitions, over a full-
     causal layer and a chunked one, checked at every step against the oracle."""
     cfg = oracle.make_config(width=64, vocab=37, layers=[
         oracle.make_layer(heads=4, kv_heads=2, dim=32, chunk=0, rot_dims=16, scaling=SCALING),
@@ -97,3 +97,20 @@ def test_greedy_generation(model):
             row = logits[len(p) - 1 + i]
             assert row[tok] >= row.max() - 1e-3 * row.std(), (i, tok, int(row.argmax()))
     assert torch.cuda.is_available()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(__import__("test_bidetar").OTHER))
+def test_other_configurations(tmp_path, name, dtype):
+    """Sizes that leave the 16-byte and matrix-core paths (odd widths, head sizes 6 / 10 / 24,
+    a 7-wide feed-forward, chunk 1): the scalar and row kernels, in mixed steps and decode."""
+    from test_bidetar import OTHER
+
+    cfg = oracle.make_config(**dict(OTHER[name]))
+    W = oracle.random_weights(cfg, seed=len(name))
+    reqs = {"p": tokens(45, cfg["vocab"], 11), "q": tokens(38, cfg["vocab"], 12)}
+    want = {n: oracle.forward(cfg, W, t)[0] for n, t in reqs.items()}
+    eng = engine(write_model(tmp_path, cfg, W), dtype=dtype, device="cuda")
+    sched = [[("p", 17), ("q", 2)], [("p", 1), ("q", 30)], [("p", 27), ("q", 1)],
+             [("q", 1)], [("q", 4)]]
+    check(replay(eng, reqs, sched), want, dtype)
