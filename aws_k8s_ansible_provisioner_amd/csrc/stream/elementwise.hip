@@ -89,8 +89,9 @@ void launch_embed_scaled(float* out, const int64_t* ids, const void* table, bool
 template <typename TY, typename TO, int NR>
 __global__ __launch_bounds__(256) void add_norm_kernel(TO* __restrict__ out, float* __restrict__ x,
                                                        const TY* __restrict__ y, int y_stride,
-                                                       float mult, const float* __restrict__ w,
-                                                       int d, int out_stride, float eps) {
+                                                       const TY* __restrict__ bias, float mult,
+                                                       const float* __restrict__ w, int d,
+                                                       int out_stride, float eps) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   float* xr = x + (size_t)row * d;
@@ -104,7 +105,7 @@ __global__ __launch_bounds__(256) void add_norm_kernel(TO* __restrict__ out, flo
     if (c < d) {
       float f = xr[c];
       if (yr) {
-        f += mult * ldf(yr + c);
+        f += mult * (ldf(yr + c) + (bias ? ldf(bias + c) : 0.f));
         xr[c] = f;
       }
       v[i] = f;
@@ -115,7 +116,7 @@ __global__ __launch_bounds__(256) void add_norm_kernel(TO* __restrict__ out, flo
   for (int c = NR * 256 + threadIdx.x; c < d; c += 256) {
     float f = xr[c];
     if (yr) {
-      f += mult * ldf(yr + c);
+      f += mult * (ldf(yr + c) + (bias ? ldf(bias + c) : 0.f));
       xr[c] = f;
     }
     ss += f * f;
@@ -137,8 +138,9 @@ template <typename TY, typename TO, int NR>
 __global__ __launch_bounds__(256) void add_norm_vec_kernel(TO* __restrict__ out,
                                                            float* __restrict__ x,
                                                            const TY* __restrict__ y, int y_stride,
-                                                           float mult, const float* __restrict__ w,
-                                                           int d, int out_stride, float eps) {
+                                                           const TY* __restrict__ bias, float mult,
+                                                           const float* __restrict__ w, int d,
+                                                           int out_stride, float eps) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   float* xr = x + (size_t)row * d;
@@ -153,6 +155,12 @@ __global__ __launch_bounds__(256) void add_norm_vec_kernel(TO* __restrict__ out,
       if (yr) {
         float yy[4];
         ldv(yy, yr + c);
+        if (bias) {
+          float bb[4];
+          ldv(bb, bias + c);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) yy[e] += bb[e];
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[i][e] += mult * yy[e];
         stv(xr + c, v[i]);
@@ -178,15 +186,16 @@ __global__ __launch_bounds__(256) void add_norm_vec_kernel(TO* __restrict__ out,
 }
 
 template <typename TY, typename TO>
-static void add_norm_t(void* out, float* x, const void* y, int y_stride, float mult,
-                       const float* w, int rows, int d, int out_stride, float eps, hipStream_t s) {
+static void add_norm_t(void* out, float* x, const void* y, int y_stride, const void* bias,
+                       float mult, const float* w, int rows, int d, int out_stride, float eps,
+                       hipStream_t s) {
   const bool vec = d % 4 == 0 && d <= 8192 && y_stride % 4 == 0 && out_stride % 4 == 0 &&
                    aligned(x, 16) && aligned(w, 16) && aligned(y, 4 * sizeof(TY)) &&
-                   aligned(out, 4 * sizeof(TO));
+                   aligned(bias, 4 * sizeof(TY)) && aligned(out, 4 * sizeof(TO));
   if (vec) {
 #define AKAP_ADD_NORM_VEC(NR)                                                                  \
-  add_norm_vec_kernel<TY, TO, NR><<<rows, 256, 0, s>>>((TO*)out, x, (const TY*)y, y_stride, mult, \
-                                                       w, d, out_stride, eps)
+  add_norm_vec_kernel<TY, TO, NR><<<rows, 256, 0, s>>>((TO*)out, x, (const TY*)y, y_stride,      \
+                                                       (const TY*)bias, mult, w, d, out_stride, eps)
     if (d <= 1024) AKAP_ADD_NORM_VEC(1);
     else if (d <= 2048) AKAP_ADD_NORM_VEC(2);
     else if (d <= 4096) AKAP_ADD_NORM_VEC(4);
@@ -195,25 +204,25 @@ static void add_norm_t(void* out, float* x, const void* y, int y_stride, float m
     return;
   }
   if (d <= 1024)
-    add_norm_kernel<TY, TO, 4><<<rows, 256, 0, s>>>((TO*)out, x, (const TY*)y, y_stride, mult, w, d,
-                                                    out_stride, eps);
+    add_norm_kernel<TY, TO, 4><<<rows, 256, 0, s>>>((TO*)out, x, (const TY*)y, y_stride,
+                                                    (const TY*)bias, mult, w, d, out_stride, eps);
   else
-    add_norm_kernel<TY, TO, 16><<<rows, 256, 0, s>>>((TO*)out, x, (const TY*)y, y_stride, mult, w,
-                                                     d, out_stride, eps);
+    add_norm_kernel<TY, TO, 16><<<rows, 256, 0, s>>>((TO*)out, x, (const TY*)y, y_stride,
+                                                     (const TY*)bias, mult, w, d, out_stride, eps);
 }
 
 void launch_add_norm(void* out, bool out_f32, float* x, const void* y, bool y_f32, int y_stride,
-                     float mult, const float* w, int rows, int d, int out_stride, float eps,
-                     hipStream_t s) {
+                     const void* bias, float mult, const float* w, int rows, int d,
+                     int out_stride, float eps, hipStream_t s) {
   if (rows <= 0) return;
   if (out_f32 && y_f32)
-    add_norm_t<float, float>(out, x, y, y_stride, mult, w, rows, d, out_stride, eps, s);
+    add_norm_t<float, float>(out, x, y, y_stride, bias, mult, w, rows, d, out_stride, eps, s);
   else if (out_f32)
-    add_norm_t<bf16, float>(out, x, y, y_stride, mult, w, rows, d, out_stride, eps, s);
+    add_norm_t<bf16, float>(out, x, y, y_stride, bias, mult, w, rows, d, out_stride, eps, s);
   else if (y_f32)
-    add_norm_t<float, bf16>(out, x, y, y_stride, mult, w, rows, d, out_stride, eps, s);
+    add_norm_t<float, bf16>(out, x, y, y_stride, bias, mult, w, rows, d, out_stride, eps, s);
   else
-    add_norm_t<bf16, bf16>(out, x, y, y_stride, mult, w, rows, d, out_stride, eps, s);
+    add_norm_t<bf16, bf16>(out, x, y, y_stride, bias, mult, w, rows, d, out_stride, eps, s);
 }
 
 template <typename T>
@@ -277,13 +286,17 @@ __global__ __launch_bounds__(256) void proj_norm_rope_cache_kernel(ProjParams p)
   const T* qr = row + p.q_off;
   const T* kr = row + p.k_off;
   const int HD = p.H * p.D, GD = p.G * p.D;
+  const T* qb = (const T*)p.q_b;
+  const T* kb = (const T*)p.k_b;
+  auto qv = [&](int c) { return ldf(qr + c) + (qb ? ldf(qb + c) : 0.f); };
+  auto kv = [&](int c) { return ldf(kr + c) + (kb ? ldf(kb + c) : 0.f); };
   float sq = 0.f, sk = 0.f;
   for (int c = threadIdx.x; c < HD; c += 256) {
-    const float f = ldf(qr + c);
+    const float f = qv(c);
     sq += f * f;
   }
   for (int c = threadIdx.x; c < GD; c += 256) {
-    const float f = ldf(kr + c);
+    const float f = kv(c);
     sk += f * f;
   }
   sq = block_sum(sq, scratch);
@@ -299,8 +312,8 @@ __global__ __launch_bounds__(256) void proj_norm_rope_cache_kernel(ProjParams p)
   for (int e = threadIdx.x; e < (HD >> 1); e += 256) {
     const int i = e % half;
     const int c = (e / half) * p.D + 2 * i;
-    float u = ldf(qr + c) * iq * p.q_w[c];
-    float v = ldf(qr + c + 1) * iq * p.q_w[c + 1];
+    float u = qv(c) * iq * p.q_w[c];
+    float v = qv(c + 1) * iq * p.q_w[c + 1];
     if (cs && i < rh) {
       const float co = cs[i], si = cs[rh + i];
       const float ru = u * co - v * si;
@@ -318,7 +331,7 @@ __global__ __launch_bounds__(256) void proj_norm_rope_cache_kernel(ProjParams p)
     const int i = e % half;
     const int g = e / half;
     const int c = g * p.D + 2 * i;
-    const float ru = ldf(kr + c), rv = ldf(kr + c + 1);
+    const float ru = kv(c), rv = kv(c + 1);
     float u = ru * ik * p.k_w[c];
     float v = rv * ik * p.k_w[c + 1];
     if (cs && i < rh) {
@@ -333,8 +346,8 @@ __global__ __launch_bounds__(256) void proj_norm_rope_cache_kernel(ProjParams p)
     // the values are the projected keys, untouched; V cache [NB, G, BS/8, D, 8]
     T* vc = (T*)p.v_cache +
             ((((size_t)blk * p.G + g) * (p.BS >> 3) + (off >> 3)) * p.D + 2 * i) * 8 + (off & 7);
-    vc[0] = kr[c];
-    vc[8] = kr[c + 1];
+    vc[0] = (T)ru;
+    vc[8] = (T)rv;
   }
 }
 
@@ -356,6 +369,12 @@ __global__ __launch_bounds__(256) void proj_norm_rope_cache_vec_kernel(ProjParam
     const int c = (i * 256 + threadIdx.x) * 8;
     if (c < HD) {
       ldv(q[i], qr + c);
+      if (p.q_b) {
+        float bb[8];
+        ldv(bb, (const T*)p.q_b + c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) q[i][e] += bb[e];
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) sq += q[i][e] * q[i][e];
     }
@@ -363,6 +382,12 @@ __global__ __launch_bounds__(256) void proj_norm_rope_cache_vec_kernel(ProjParam
   const int ck = threadIdx.x * 8;
   if (ck < GD) {
     ldv(k, kr + ck);
+    if (p.k_b) {
+      float bb[8];
+      ldv(bb, (const T*)p.k_b + ck);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) k[e] += bb[e];
+    }
 #pragma unroll
     for (int e = 0; e < 8; ++e) sk += k[e] * k[e];
   }
@@ -413,7 +438,7 @@ __global__ __launch_bounds__(256) void proj_norm_rope_cache_vec_kernel(ProjParam
   for (int c = threadIdx.x; c < GD; c += 256) {
     const int g = c / p.D, d = c - g * p.D;
     ((T*)p.v_cache)[((((size_t)blk * p.G + g) * (p.BS >> 3) + (off >> 3)) * p.D + d) * 8 +
-                    (off & 7)] = kr[c];
+                    (off & 7)] = (T)(ldf(kr + c) + (p.k_b ? ldf((const T*)p.k_b + c) : 0.f));
   }
   if (ck >= GD) return;
   const int g = ck / p.D, d0 = ck % p.D;
@@ -426,6 +451,7 @@ static bool proj_vec_ok(const ProjParams& p) {
   const size_t a = 8 * sizeof(T) > 16 ? 16 : 8 * sizeof(T);
   return p.D % 8 == 0 && p.q_off % 8 == 0 && p.k_off % 8 == 0 && p.proj_stride % 8 == 0 &&
          p.H * p.D <= 4096 && p.G * p.D <= 2048 && aligned(p.proj, a) && aligned(p.q_out, a) &&
+         aligned(p.q_b, a) && aligned(p.k_b, a) &&
          aligned(p.k_cache, a) && aligned(p.q_w, 16) && aligned(p.k_w, 16);
 }
 

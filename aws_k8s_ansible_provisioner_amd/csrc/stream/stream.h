@@ -13,9 +13,10 @@ namespace akap_stream {
 void launch_embed_scaled(float* out, const int64_t* ids, const void* table, bool f32, int rows,
                          int d, int vocab, float scale, hipStream_t s);
 // x (fp32, contiguous rows of d) += mult * y (y may be null); out = rmsnorm(x) * w
+// (bias: d values of y's type added to every row of y, or null)
 void launch_add_norm(void* out, bool out_f32, float* x, const void* y, bool y_f32, int y_stride,
-                     float mult, const float* w, int rows, int d, int out_stride, float eps,
-                     hipStream_t s);
+                     const void* bias, float mult, const float* w, int rows, int d,
+                     int out_stride, float eps, hipStream_t s);
 void launch_relu2(void* out, const void* x, bool f32, int rows, int F, int x_stride,
                   int out_stride, hipStream_t s);
 
@@ -31,6 +32,8 @@ struct ProjParams {
   int max_pos, rot_dims;
   const float* q_w;      // [H D]
   const float* k_w;      // [G D]
+  const void* q_b;       // [H D] / [G D] of the projection's type, added to the q / k slices
+  const void* k_b;       //   before anything else (the projection's biases), or null
   int T, H, G, D, BS, q_off, k_off;
   int64_t num_slots;     // NB * BS
   float eps;

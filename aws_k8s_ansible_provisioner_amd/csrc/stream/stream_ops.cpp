@@ -40,7 +40,8 @@ void embed_scaled(Tensor out, Tensor ids, Tensor table, double scale) {
                                    (int)table.size(0), (float)scale, cur_stream());
 }
 
-void add_norm(Tensor out, Tensor x, std::optional<Tensor> y, double mult, Tensor w, double eps) {
+void add_norm(Tensor out, Tensor x, std::optional<Tensor> y, double mult, Tensor w, double eps,
+              std::optional<Tensor> bias) {
   CHECK_GPU(out); CHECK_GPU(x); CHECK_GPU(w);
   CHECK_F32(x); CHECK_CONTIG(x); CHECK_F32(w); CHECK_CONTIG(w); CHECK_LAST_CONTIG(out);
   TORCH_CHECK(x.dim() == 2 && out.dim() == 2 && out.sizes() == x.sizes(), "add_norm: shapes");
@@ -56,9 +57,17 @@ void add_norm(Tensor out, Tensor x, std::optional<Tensor> y, double mult, Tensor
     yf = is_f32(*y, "y");
     ys = y->stride(0);
   }
+  const void* bp = nullptr;
+  if (bias.has_value()) {
+    TORCH_CHECK(y.has_value(), "add_norm: a bias needs y");
+    CHECK_GPU(*bias); CHECK_CONTIG(*bias);
+    TORCH_CHECK(bias->numel() == d && bias->scalar_type() == y->scalar_type(),
+                "add_norm: bias must be [d] of y's dtype");
+    bp = bias->data_ptr();
+  }
   const c10::DeviceGuard g(x.device());
   akap_stream::launch_add_norm(out.data_ptr(), is_f32(out, "out"), x.data_ptr<float>(), yp, yf, ys,
-                               (float)mult, w.data_ptr<float>(), rows, d, (int)out.stride(0),
+                               bp, (float)mult, w.data_ptr<float>(), rows, d, (int)out.stride(0),
                                (float)eps, cur_stream());
 }
 
@@ -86,7 +95,8 @@ void check_cache(const Tensor& k_cache, const Tensor& v_cache, int64_t G, int64_
 void proj_norm_rope_cache(Tensor proj, Tensor q_out, Tensor k_cache, Tensor v_cache,
                           Tensor positions, Tensor slots, std::optional<Tensor> cos_sin,
                           Tensor q_w, Tensor k_w, int64_t H, int64_t G, int64_t D, int64_t q_off,
-                          int64_t k_off, double eps) {
+                          int64_t k_off, double eps, std::optional<Tensor> q_b,
+                          std::optional<Tensor> k_b) {
   CHECK_GPU(proj); CHECK_LAST_CONTIG(proj); CHECK_GPU(q_out); CHECK_CONTIG(q_out);
   CHECK_GPU(positions); CHECK_GPU(slots); CHECK_GPU(q_w); CHECK_GPU(k_w);
   CHECK_F32(q_w); CHECK_F32(k_w); CHECK_CONTIG(q_w); CHECK_CONTIG(k_w);
@@ -112,6 +122,16 @@ void proj_norm_rope_cache(Tensor proj, Tensor q_out, Tensor k_cache, Tensor v_ca
     p.cos_sin = cos_sin->data_ptr<float>();
     p.max_pos = cos_sin->size(0);
     p.rot_dims = cos_sin->size(1);
+  }
+  if (q_b.has_value()) {
+    CHECK_GPU(*q_b); CHECK_CONTIG(*q_b);
+    TORCH_CHECK(q_b->numel() == H * D && q_b->scalar_type() == proj.scalar_type(), "q_b: [H D]");
+    p.q_b = q_b->data_ptr();
+  }
+  if (k_b.has_value()) {
+    CHECK_GPU(*k_b); CHECK_CONTIG(*k_b);
+    TORCH_CHECK(k_b->numel() == G * D && k_b->scalar_type() == proj.scalar_type(), "k_b: [G D]");
+    p.k_b = k_b->data_ptr();
   }
   p.proj = proj.data_ptr();
   p.proj_stride = proj.stride(0);
@@ -231,12 +251,13 @@ void sink_attention_decode(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
 
 TORCH_LIBRARY(akap_stream, m) {
   m.def("embed_scaled(Tensor(a!) out, Tensor ids, Tensor table, float scale) -> ()");
-  m.def("add_norm(Tensor(a!) out, Tensor(b!) x, Tensor? y, float mult, Tensor w, float eps) -> ()");
+  m.def("add_norm(Tensor(a!) out, Tensor(b!) x, Tensor? y, float mult, Tensor w, float eps, "
+        "Tensor? bias=None) -> ()");
   m.def("relu2(Tensor(a!) out, Tensor x) -> ()");
   m.def(
       "proj_norm_rope_cache(Tensor proj, Tensor(a!) q_out, Tensor(b!) k_cache, Tensor(c!) v_cache, "
       "Tensor positions, Tensor slots, Tensor? cos_sin, Tensor q_w, Tensor k_w, int H, int G, "
-      "int D, int q_off, int k_off, float eps) -> ()");
+      "int D, int q_off, int k_off, float eps, Tensor? q_b=None, Tensor? k_b=None) -> ()");
   m.def(
       "sink_attention_prefill(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
       "Tensor block_tables, Tensor seq_lens, Tensor q_start, Tensor tile_seq, Tensor tile_row, "

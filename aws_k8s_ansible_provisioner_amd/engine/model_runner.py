@@ -56,10 +56,11 @@ class ModelRunner:
         self.log = log
         dev = ecfg.resolved_device()
         cls = model_class(mcfg)
-        # models on the stream kernels (ops.stream) need the core library only for the sampler
-        # and the staging kernel: a step that returns logits alone runs without it
-        self._core_native = dev == "cuda" and (getattr(cls, "gemm_tunable", True)
-                                               or not ecfg.logits_only)
+        # models on the stream kernels (ops.stream) need the core library for the sampler, the
+        # staging kernel and the tuned decode GEMMs: a replay engine that returns logits alone
+        # (a handful of sequence slots, library GEMMs) runs without building or loading it
+        self._core_native = dev == "cuda" and not (
+            ecfg.logits_only and getattr(cls, "prefill_tile_plan", None) is not None)
         if dev == "cuda":
             self.device = torch.device("cuda", torch.cuda.current_device())
             if self._core_native:
@@ -793,7 +794,7 @@ class ModelRunner:
                 "AKAP_TUNABLEOP_FILE", os.path.join(os.getcwd(), "tunableop_results.csv")))
         # safe static contents: every row is padding
         self._pad_host(0, self.max_seqs)
-        if os.environ.get("AKAP_GEMM_TUNE", "1") != "0" and \
+        if os.environ.get("AKAP_GEMM_TUNE", "1") != "0" and self._core_native and \
                 getattr(self.model, "gemm_tunable", True):
             # MoE models: the attention projections are tuned (the experts run the grouped
             # GEMM; tune_fused skips MoE layers)
@@ -821,9 +822,12 @@ class ModelRunner:
                          f"({len(gemm_tuner.plan())} shapes)")
             else:
                 gemm_tuner.tune_model(self.model, tune_ms, log=self.log)
-                if os.environ.get("AKAP_FUSED_GEMM", "1") != "0":
+                # (the fused 4-GEMM decode chain and the hand-written prefill GEMM are planned
+                # for the dense Llama-style layer only)
+                dense = getattr(self.model, "fused_gemm_chain", True)
+                if dense and os.environ.get("AKAP_FUSED_GEMM", "1") != "0":
                     gemm_tuner.tune_fused(self.model, tune_ms, log=self.log)
-                if ops.PREFILL_GEMM == "auto" and pre_m >= ops.PGEMM_MIN_M:
+                if dense and ops.PREFILL_GEMM == "auto" and pre_m >= ops.PGEMM_MIN_M:
                     gemm_tuner.tune_prefill(self.model, pre_m, log=self.log)
                 if cache:
                     gemm_tuner.save_cache(cache, self.model, tune_ms, pre_m)

@@ -26,6 +26,7 @@ from typing import Optional
 import torch
 import torch.nn.functional as F
 
+from .. import ops
 from ..ops import stream as sops
 from ..parallel.state import ParallelState, get_state
 from .config import LayeredConfig, LayerSpec
@@ -58,7 +59,12 @@ class BidetarLM:
     """Weights + forward of one replica (same surface as DecoderLM for the model runner)."""
 
     supports_v_tail = False   # the D = 128 decode kernel's V-group tail is not used here
-    gemm_tunable = False      # projections go to hipBLASLt; no decode-GEMM plan to tune
+    # the two per-layer GEMM weights: decode-sized batches are tuned per shape like the other
+    # models' projections (ops.gemm_tuner: the MFMA decode kernels against hipBLASLt); there is
+    # no fused 4-GEMM decode chain and no hand-written prefill GEMM plan for this layer shape
+    gemm_tunable = True
+    gemm_weight_names = ("w_in", "w_out")
+    fused_gemm_chain = False
     dtypes = (torch.bfloat16, torch.float32)
 
     def __init__(self, cfg: LayeredConfig, device: torch.device | str = "cpu",
@@ -116,7 +122,11 @@ class BidetarLM:
             hd, gd = m.heads * m.dim, m.kv_heads * m.dim
             ff = ls.mlp.ff if ls.mlp is not None else 0
             n = hd + gd + ff + m.heads
-            npad = -(-n // 8) * 8
+            # rows padded (zeros) to the tile width of the decode GEMM kernels when that costs
+            # under 5 %, else to whole 16-byte rows of the output
+            npad = -(-n // 256) * 256
+            if npad > 1.05 * n:
+                npad = -(-n // 8) * 8
             w_in = torch.zeros(npad, d, dtype=self.dtype, device=self.device)
             b_in = torch.zeros(npad, dtype=self.dtype, device=self.device)
             w_in[:n] = rand(n, d)
@@ -253,6 +263,13 @@ class BidetarLM:
             self._ws = (need, sops.decode_workspace(rows, self.hq, self.D, parts, self.device))
         return self._ws[1]
 
+    def _linear(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        """x @ w.T: bf16 goes through ops.linear (the tuned decode GEMM of this shape when the
+        runner tuned one, else hipBLASLt); fp32 always to the library."""
+        if self.dtype == torch.bfloat16:
+            return ops.linear(x, w)
+        return F.linear(x, w)
+
     def embed_tokens(self, ids: torch.Tensor) -> torch.Tensor:
         return sops.embed_scaled(ids, self.embed, self.cfg.embed_scale)
 
@@ -282,20 +299,22 @@ class BidetarLM:
         for r, li in enumerate(self.runs):
             lw = self.layers[li]
             m = lw.spec.mixer
-            proj = F.linear(h, lw.w_in, lw.b_in)             # [T, q | k | up | gate]
+            # [T, q | k | up | gate]; the q / k biases are added by the kernel that reads them
+            proj = self._linear(h, lw.w_in)
             q = torch.empty(T, m.heads, m.dim, dtype=dt, device=self.device)
             sops.proj_norm_rope_cache(proj, q, k_caches[r], v_caches[r], batch.positions,
                                       batch.slots, lw.cos_sin, lw.q_norm, lw.k_norm, m.heads,
-                                      m.kv_heads, m.dim, 0, lw.k_off, eps)
+                                      m.kv_heads, m.dim, 0, lw.k_off, eps,
+                                      lw.b_in[:lw.hd], lw.b_in[lw.k_off:lw.up_off])
             cat = torch.empty(T, lw.hd + lw.ff, dtype=dt, device=self.device)
             gate = proj[:, lw.g_off:lw.g_off + m.heads] if m.gate else None
             self._attention(lw, q, gate, batch, k_caches[r], v_caches[r], cat)
             if lw.ff:
                 sops.relu2(proj[:, lw.up_off:lw.g_off], cat[:, lw.hd:])
-            y = F.linear(cat, lw.w_out, lw.b_out)            # W_o attn + W_down act + b_o
+            y = self._linear(cat, lw.w_out)                  # W_o attn + W_down act
             nxt = self.layers[self.runs[r + 1]].norm1 if r + 1 < len(self.runs) \
                 else self.final_norm
-            h = sops.stream_add_norm(x, y, mult, nxt, eps, dt)
+            h = sops.stream_add_norm(x, y, mult, nxt, eps, dt, bias=lw.b_out)   # ... + b_o
         return h
 
     def compute_logits(self, h: torch.Tensor) -> torch.Tensor:

@@ -280,11 +280,19 @@ def _gd_name(v) -> str:
     return f"g{bn}" + ("d" if ns >= 6 else "") + ("i" if inl else "")
 
 
+DENSE_WEIGHTS = ("w_qkv", "w_o", "w_gate_up", "w_down")
+
+
+def weight_names(model) -> tuple:
+    """The per-layer GEMM weight attributes of a model (its own list, or the dense layer's)."""
+    return tuple(getattr(model, "gemm_weight_names", DENSE_WEIGHTS))
+
+
 def tune_model(model, Ms: Sequence[int], log=print) -> dict:
     """Tune every dense projection shape of `model` (per layer type) for each M."""
     groups = {}
     for lw in model.layers:
-        for name in ("w_qkv", "w_o", "w_gate_up", "w_down"):
+        for name in weight_names(model):
             w = getattr(lw, name, None)
             if w is not None:
                 groups.setdefault((name, tuple(w.shape)), []).append(w)
@@ -568,7 +576,7 @@ def cache_key(model, Ms: Sequence[int], prefill_m: int = 0) -> dict:
     from . import _LIB
 
     shapes = sorted({(name, tuple(getattr(lw, name).shape)) for lw in model.layers
-                     for name in ("w_qkv", "w_o", "w_gate_up", "w_down")
+                     for name in weight_names(model)
                      if getattr(lw, name, None) is not None})
     lm = getattr(model, "lm_head", None)
     try:

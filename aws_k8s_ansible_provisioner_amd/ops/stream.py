@@ -84,15 +84,17 @@ def stream_norm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype: torch.d
 
 
 def stream_add_norm(x: torch.Tensor, y: torch.Tensor, mult: float, w: torch.Tensor, eps: float,
-                    out_dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x += mult * y in place (fp32 sum), then the RMS norm of the new x as out_dtype: the
-    residual update of one layer fused with the norm that feeds the next."""
+                    out_dtype: torch.dtype, out: Optional[torch.Tensor] = None,
+                    bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x += mult * (y + bias) in place (fp32 sum), then the RMS norm of the new x as out_dtype:
+    the residual update of one layer fused with the norm that feeds the next.  bias [d] (y's
+    dtype): the bias of the projection that produced y, when its GEMM has no bias epilogue."""
     if out is None:
         out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
     if _native(x):
-        torch.ops.akap_stream.add_norm(out, x, y, float(mult), w, float(eps))
+        torch.ops.akap_stream.add_norm(out, x, y, float(mult), w, float(eps), bias)
         return out
-    x.add_(y.float() * mult)
+    x.add_((y.float() + (bias.float() if bias is not None else 0.0)) * mult)
     out.copy_((_rms(x, eps) * w.float()).to(out.dtype))
     return out
 
@@ -127,22 +129,29 @@ def rotary_table(max_pos: int, dims: int, base: float, scaling: Optional[dict] =
 def proj_norm_rope_cache(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor,
                          v_cache: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor,
                          cos_sin: Optional[torch.Tensor], q_w: torch.Tensor, k_w: torch.Tensor,
-                         H: int, G: int, D: int, q_off: int, k_off: int, eps: float) -> None:
+                         H: int, G: int, D: int, q_off: int, k_off: int, eps: float,
+                         q_b: Optional[torch.Tensor] = None,
+                         k_b: Optional[torch.Tensor] = None) -> None:
     """Per token t of the fused projection proj [T, N]: q = proj[t, q_off : q_off + H D] and
     k = proj[t, k_off : k_off + G D] are each RMS-normalised over their WHOLE length (one
     mean over all heads) with weights q_w / k_w, then rotated per head on the first
     cos_sin.shape[1] dimensions, interleaved pairs (2i, 2i+1), by the angle row of
     positions[t].  q goes to q_out [T, H, D]; k to k_cache at slots[t]; the raw k (before norm
     and rotation) to v_cache at the same slot: the values are the keys' projection.  Slot -1
-    writes nothing.  k_cache [NB, G, BS, D], v_cache [NB, G, BS/8, D, 8]."""
+    writes nothing.  k_cache [NB, G, BS, D], v_cache [NB, G, BS/8, D, 8].  q_b / k_b (proj's
+    dtype): the projection's biases, added to the slices first when its GEMM did not."""
     if _native(proj):
         torch.ops.akap_stream.proj_norm_rope_cache(proj, q_out, k_cache, v_cache, positions, slots,
                                                    cos_sin, q_w, k_w, H, G, D, q_off, k_off,
-                                                   float(eps))
+                                                   float(eps), q_b, k_b)
         return
     T = proj.shape[0]
     q = proj[:, q_off:q_off + H * D].float()
     k = proj[:, k_off:k_off + G * D].float()
+    if q_b is not None:
+        q = q + q_b.float()
+    if k_b is not None:
+        k = k + k_b.float()
     qn = (_rms(q, eps) * q_w.float()).view(T, H, D)
     kn = (_rms(k, eps) * k_w.float()).view(T, G, D)
     if cos_sin is not None:
