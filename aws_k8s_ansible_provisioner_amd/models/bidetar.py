@@ -9,13 +9,16 @@ output gate.  The feed-forward is down(relu(up h)^2).  A span of layers may run 
 in a row with the same weights; every pass has its own KV cache.
 
 MI355X mapping: the parallel layer collapses to TWO GEMMs.  All projections that read h are one
-weight [q | k | up | gate] and one hipBLASLt launch; the attention output and the activated
-feed-forward share one buffer [attn | act] that a single GEMM with the weight [W_o | W_down]
-reduces (the sum of the two sublayers happens in the GEMM's fp32 accumulator).  Between them:
-one kernel norms + rotates q and k and writes the paged cache, one attention kernel (prefill
-tiles or split decode) applies mask, sink and gate, one activation kernel; the residual update
-and the next layer's norm are one kernel on the fp32 stream.  Seven launches per layer, all
-sync-free and allocation-stable, so the runner captures decode steps in hipGraphs.
+weight [q | k | up | gate] and one launch; the attention output and the activated feed-forward
+share one buffer [attn | act] that a single GEMM with the weight [W_o | W_down] reduces (the
+sum of the two sublayers happens in the GEMM's fp32 accumulator).  Neither GEMM has a bias
+epilogue -- the q / k biases are added by the kernel that norms them, the output bias by the
+residual kernel -- so decode-sized batches run the per-shape tuned MFMA GEMMs and prefill-sized
+ones hipBLASLt, through ops.linear like every other model.  Between the GEMMs: one kernel
+norms + rotates q and k and writes the paged cache, one attention kernel (prefill tiles or
+split decode) applies mask, sink and gate, one activation kernel; the residual update and the
+next layer's norm are one kernel on the fp32 stream.  Seven launches per layer, all sync-free
+and allocation-stable, so the runner captures decode steps in hipGraphs.
 """
 from __future__ import annotations
 
