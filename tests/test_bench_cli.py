@@ -110,7 +110,7 @@ def test_bench_gpus_n_without_launcher_starts_n_ranks():
 
 def test_bench_compare_design_option():
     """--compare-design prints one JSON line with prefill and decode throughput per model and
-    leaves the default contract alone."""
+    leaves the default output alone."""
     cmd = [sys.executable, os.path.join(REPO, "bench.py"), "--compare-design", "bidetar",
            "--compare-models", "tiny-bidetar,tiny-llama", "--device", "cpu", "--steps", "1"]
     r = subprocess.run(cmd, capture_output=True, text=True, timeout=420, cwd="/tmp")
