@@ -184,14 +184,17 @@ __device__ __forceinline__ void finish_row(const Softmax& st, const AttnParams& 
   }
 }
 
-// grid (tiles, H); 4 waves share a tile's tokens
+// grid (tiles x H, flat); 4 waves share a tile's tokens
 template <typename T>
 __global__ __launch_bounds__(256) void sink_attn_prefill_rows_kernel(AttnParams p) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6;
   float* qs = smem + wave * (p.D + 64);
   float* ps = qs + p.D;
-  const int tile = blockIdx.x, h = blockIdx.y;
+  // flat grid, walked from the END of the tile map: the scheduler sorts tiles by ascending
+  // causal work, so the longest tiles start first and the shortest fill the tail; the heads of
+  // a tile (and of a GQA group) are neighbours and share its K / V in L2
+  const int tile = p.num_tiles - 1 - (int)(blockIdx.x / p.H), h = (int)(blockIdx.x % p.H);
   const int b = p.tile_seq[tile];
   if (b < 0 || b >= p.B) return;
   const int r0 = p.tile_row[tile];
@@ -493,14 +496,24 @@ __device__ __forceinline__ void mfma_finish(const MfmaState<DB, NQ>& st, int q,
       o[32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = (bf16)(st.o[q][dt][i] * f);
 }
 
-// Prefill: grid (tiles of 128 or 256 tokens, H), tile / (32 NQ) waves of NQ column tiles each.
+// Prefill: grid (tiles of 128 or 256 tokens x H, flat), tile / (32 NQ) waves of NQ column tiles each.
 template <int DB, int NQ>
 __global__ __launch_bounds__(512 / NQ) void sink_attn_prefill_mfma_kernel(AttnParams p) {
   constexpr int D = 32 * DB, KS = 2 * DB;
   using akap::bf16x8;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int col = lane & 31, hf = lane >> 5;
-  const int tile = blockIdx.x, h = blockIdx.y;
+  // Flat grid.  Work units are (tile, K/V head) pairs, taken from the END of the tile map: the
+  // scheduler sorts tiles by ascending causal work, so the longest start first and the
+  // shortest fill the tail.  The hardware deals workgroup i to XCD i % 8: units are dealt
+  // round-robin over the XCDs in that order (balanced), and the query heads of one unit are
+  // consecutive workgroups of ONE XCD, so a GQA group's K / V crosses into a single L2.
+  const int rep = p.H / p.G;
+  const int xcd = blockIdx.x & 7, jx = blockIdx.x >> 3;
+  const int unit = (jx / rep) * 8 + xcd;
+  if (unit >= p.num_tiles * p.G) return;
+  const int tile = p.num_tiles - 1 - unit / p.G;
+  const int h = (unit % p.G) * rep + jx % rep;
   const int b = p.tile_seq[tile];
   if (b < 0 || b >= p.B) return;
   const int qs0 = p.q_start[b];
@@ -606,8 +619,10 @@ static bool mfma_ok(const AttnParams& p, bool f32) {
 
 void launch_sink_attention_prefill(const AttnParams& p, bool f32, hipStream_t s) {
   if (p.num_tiles <= 0) return;
-  const dim3 grid(p.num_tiles, p.H);
+  const dim3 grid((unsigned)p.num_tiles * p.H);
   if (mfma_ok(p, f32) && (p.tile_rows == 128 || p.tile_rows == 256)) {
+    // (tile, K/V head) units padded to a multiple of the 8 XCDs, rep workgroups each
+    const dim3 grid((unsigned)((p.num_tiles * p.G + 7) / 8 * 8) * (p.H / p.G));
     const int tr = p.tile_rows;
     static const int nq = [] {  // AKAP_STREAM_NQ=1|2: column tiles per wave (A/B knob)
       const char* e = getenv("AKAP_STREAM_NQ");
