@@ -369,3 +369,44 @@ def test_greedy_generation_through_the_engine(model):
         for i, tok in enumerate(o.output_ids):
             row = logits[len(p) - 1 + i]
             assert row[tok] >= row.max() - 1e-3 * row.std(), (i, tok, int(row.argmax()))
+
+
+def test_trace_run_command_line(model, reference, tmp_path):
+    """bin/trace_run: JSON steps on stdin, one `done <step>` line per step, `<step>.f32` with
+    the logits of the wanted places (entries' order, then each entry's `want` order)."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    cfg, _, path = model
+    reqs, want = reference
+    a, c = reqs["a"], reqs["c"]
+    steps = [
+        {"step": 0, "entries": [{"id": "x", "tokens": a[:40], "want": [39, 0, 7]},
+                                {"id": "y", "tokens": c[:1], "want": [0]}], "end": []},
+        {"step": 1, "entries": [{"id": "y", "tokens": c[1:], "want": []}], "end": ["y"]},
+        {"step": 2, "entries": [{"id": "x", "tokens": a[40:41], "want": [0]}], "end": []},
+        {"step": 3, "entries": [{"id": "x", "tokens": a[41:], "want": [33]},
+                                {"id": "z", "tokens": c, "want": [22, 21]}], "end": ["x", "z"]},
+    ]
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    r = subprocess.run([sys.executable, os.path.join(repo, "bin", "trace_run"), "--model", path,
+                        "--dtype", "float32", "--out", str(out), "--max-tokens", "192",
+                        "--device", "cpu"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True,
+                       text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [ln for ln in r.stdout.splitlines() if ln.startswith("done")] == \
+        [f"done {i}" for i in range(4)]
+    assert sorted(os.listdir(out)) == ["0.f32", "2.f32", "3.f32"]   # nothing wanted in step 1
+    V = cfg["vocab"]
+    got0 = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V)).double()
+    exp0 = torch.stack([want["a"][39], want["a"][0], want["a"][7], want["c"][0]])
+    assert rel_err(got0, exp0).max().item() < FP32_TOL
+    got3 = torch.from_numpy(np.fromfile(out / "3.f32", dtype="<f4").reshape(-1, V)).double()
+    exp3 = torch.stack([want["a"][74], want["c"][22], want["c"][21]])
+    assert rel_err(got3, exp3).max().item() < FP32_TOL
