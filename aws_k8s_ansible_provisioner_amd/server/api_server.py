@@ -621,6 +621,8 @@ def make_parser() -> argparse.ArgumentParser:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--load-format", default="random", choices=["random", "safetensors"])
     ap.add_argument("--weights-path", default=None)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"],
+                    help="compute type (float32: models whose kernels have fp32 instantiations)")
     ap.add_argument("--kv-role", default="both", choices=["both", "prefill", "decode"])
     ap.add_argument("--pd-bootstrap", default=os.environ.get("AKAP_PD_BOOTSTRAP", "launcher"),
                     choices=["launcher", "http"],
@@ -658,7 +660,8 @@ def engine_config_from_args(a) -> EngineConfig:
         num_gpu_blocks=a.num_gpu_blocks, enable_prefix_caching=not a.no_enable_prefix_caching,
         enforce_eager=a.enforce_eager, tensor_parallel_size=a.tensor_parallel_size, seed=a.seed,
         device=a.device, load_format=a.load_format, weights_path=a.weights_path,
-        chat_template=a.chat_template, kv_role=a.kv_role, kv_cache_dtype=a.kv_cache_dtype)
+        chat_template=a.chat_template, kv_role=a.kv_role, kv_cache_dtype=a.kv_cache_dtype,
+        dtype=a.dtype)
 
 
 def pd_group_id() -> str:

@@ -192,3 +192,34 @@ def test_prefix_cache_and_queue_time_metrics_are_live():
     assert vals["vllm:prefix_cache_queries_total"] >= 2 * 99
     assert vals["vllm:prefix_cache_hits_total"] >= 96  # 3 full 32-token blocks reused
     assert vals["vllm:request_queue_time_seconds_count"] == 2
+
+
+def test_bidetar_served_with_prefix_cache_and_sampling():
+    """The layered fp32-stream design behind the same OpenAI endpoints: greedy completions are
+    reproducible, a repeated prompt reuses its cached pages (every layer run keeps its K / V
+    under the same page ids) and returns the same tokens, sampled requests run too."""
+    from fastapi.testclient import TestClient
+
+    from aws_k8s_ansible_provisioner_amd.engine.config import EngineConfig
+    from aws_k8s_ansible_provisioner_amd.server.api_server import build_app
+
+    app, ae = build_app(EngineConfig(model="tiny-bidetar", served_model_name="b", device="cpu",
+                                     dtype="float32", max_model_len=256, max_num_seqs=4,
+                                     max_num_batched_tokens=48, block_size=32,
+                                     num_gpu_blocks=64))
+    prompt = list(range(10, 110))
+    with TestClient(app) as c:
+        outs = []
+        for _ in range(2):
+            r = c.post("/v1/completions", json={"prompt": prompt, "max_tokens": 6,
+                                                "temperature": 0.0})
+            assert r.status_code == 200, r.text
+            outs.append(r.json()["choices"][0]["text"])
+        assert outs[0] == outs[1]
+        r = c.post("/v1/completions", json={"prompt": prompt[:50], "max_tokens": 5,
+                                            "temperature": 0.8, "top_p": 0.9, "seed": 3})
+        assert r.status_code == 200 and r.json()["usage"]["completion_tokens"] == 5
+        text = c.get("/metrics").text
+    hits = sum(float(ln.rsplit(" ", 1)[1]) for ln in text.splitlines()
+               if ln.startswith("vllm:prefix_cache_hits_total"))
+    assert hits >= 96  # the second request reused 3 full pages of the first
