@@ -96,7 +96,12 @@ class LLMEngine:
         sc.max_decode_stall_steps = ecfg.max_decode_stall_steps
         sc.held_kv_ttl_s = ecfg.held_kv_ttl_s
         sc.num_tail_slots = self.runner.num_tail_slots
-        self.sched = rt.Scheduler(sc, self.runner.num_blocks, ecfg.enable_prefix_caching)
+        prefix = ecfg.enable_prefix_caching
+        if prefix and getattr(self.runner.model, "state_slots", False):
+            # a cached prefix holds keys and values, not the recurrent state at its end
+            log("[engine] prefix caching is off: the model keeps per-sequence state")
+            prefix = False
+        self.sched = rt.Scheduler(sc, self.runner.num_blocks, prefix)
         self.tokenizer = get_tokenizer(ecfg.weights_path, self.mcfg.vocab_size, self.mcfg.bos_id,
                                        self.mcfg.eos_id)
         self.metrics = EngineMetrics(self.model_name)

@@ -135,6 +135,11 @@ class ModelRunner:
             self._tail = torch.zeros(mcfg.num_layers, self.num_tail_slots, self.model.hkv, 8,
                                      self.model.D, dtype=torch.bfloat16, device=self.device)
             self.v_tails = list(self._tail.unbind(0))
+        elif getattr(self.model, "state_slots", False):
+            # recurrent per-sequence state (one row set per live sequence): the same slot pool
+            # of the scheduler, held from a sequence's first step to its end and used again
+            self.num_tail_slots = self.max_seqs
+            self.model.allocate_state(self.num_tail_slots)
         # workspace sized for the finest split any bucket uses (256-token partitions)
         self.num_parts = max(1, math.ceil(ecfg.max_model_len / 128))
         self._alloc_buffers()

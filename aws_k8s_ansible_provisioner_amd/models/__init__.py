@@ -7,6 +7,10 @@ def model_class(cfg: ModelConfig):
         from .bidetar import BidetarLM
 
         return BidetarLM
+    if cfg.arch == "puputar":
+        from .puputar import PuputarLM
+
+        return PuputarLM
     from .transformer import DecoderLM
 
     return DecoderLM

@@ -18,7 +18,7 @@ from typing import Optional
 class ModelConfig:
     name: str
     hf_id: str
-    arch: str  # "qwen3" | "llama" | "mixtral" | "qwen3_moe" | "bidetar" (LayeredConfig)
+    arch: str  # "qwen3" | "llama" | "mixtral" | "qwen3_moe" | "bidetar" | "puputar" (LayeredConfig)
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -126,16 +126,69 @@ class AttentionSpec:
 
 
 @dataclasses.dataclass
+class LatentAttentionSpec:
+    """Attention through low-rank latents: queries are W_uq rms(W_dq h) (rank q_rank), keys and
+    values are up-projections (W_uk, W_uv, per head) of ONE cached latent c = rms(W_dkv h) of
+    size kv_rank, plus a rotated key part of rot_dim dimensions shared by all heads.  A head
+    has `dim` unrotated and `rot_dim` rotated query/key dimensions and values of size `vdim`.
+    gate: "head" (one sigmoid per head) or "element" (one per output dimension), computed from
+    the mixer's input.  kv_from: index of an earlier layer whose cached latent and rotated key
+    this layer reads instead of projecting its own."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    q_rank: int
+    scale: float
+    rot: RotarySpec
+    gate: str = "head"
+    kv_from: Optional[int] = None
+    # sizing fields shared with AttentionSpec: one cached "head" of kv_rank + rot_dim entries
+    kv_heads: int = 1
+    chunk: int = 0
+    window: int = 0
+
+    @property
+    def cache_dim(self) -> int:
+        return self.kv_rank + self.rot_dim
+
+    @property
+    def gate_rows(self) -> int:
+        return self.heads if self.gate == "head" else self.heads * self.vdim
+
+
+@dataclasses.dataclass
+class RouterSpec:
+    """Softmax router over experts + identity outputs (the last `identity` outputs return their
+    input).  The choice adds a per-output correction to the scores; outputs form
+    `groups` equal groups of neighbours of which only the `keep` best (by their largest
+    choice score) may be chosen from; `top` outputs are chosen and their uncorrected scores
+    renormalised."""
+    experts: int
+    top: int
+    identity: int = 0
+    groups: int = 1
+    keep: int = 1
+
+    @property
+    def outputs(self) -> int:
+        return self.experts + self.identity
+
+
+@dataclasses.dataclass
 class MlpSpec:
-    kind: str   # "dense": down(act(up h))
+    kind: str   # "dense": down(act(up h)) | "moe": routed experts of that form
     ff: int
-    act: str = "relu2"
+    act: str = "relu2"              # "relu2" | "xielu" (two learned numbers per layer)
+    bias: bool = False
+    router: Optional[RouterSpec] = None
 
 
 @dataclasses.dataclass
 class LayerSpec:
-    type: str                       # which mixer: "attention"
-    mixer: AttentionSpec
+    type: str                       # which mixer: "attention" | "latent_attention[_2]"
+    mixer: object                   # AttentionSpec | LatentAttentionSpec
     mlp: Optional[MlpSpec] = None   # None: the layer has no feed-forward
 
 
@@ -150,6 +203,7 @@ class LayeredConfig(ModelConfig):
     loop: Optional[tuple] = None    # (start, stop, times)
     embed_scale: float = 1.0
     residual_mult: float = 1.0
+    norm_groups: int = 1            # RMS norms of the stream run in this many equal parts
 
     def layer_runs(self) -> list:
         """Indices into layer_specs in execution order."""
@@ -161,14 +215,32 @@ class LayeredConfig(ModelConfig):
 
     def kv_bytes_per_token(self, tp: int = 1) -> int:
         es = 4 if self.dtype == "float32" else 2
-        return sum(2 * self.layer_specs[i].mixer.kv_heads * self.layer_specs[i].mixer.dim * es
-                   for i in self.layer_runs())
+        n = 0
+        for i in self.layer_runs():
+            m = self.layer_specs[i].mixer
+            if isinstance(m, LatentAttentionSpec):
+                n += 0 if m.kv_from is not None else m.cache_dim * es
+            else:
+                n += 2 * m.kv_heads * m.dim * es
+        return n
 
     def num_params(self) -> int:
         d = self.hidden_size
         n = 2 * self.vocab_size * d + d
         for ls in self.layer_specs:
             m = ls.mixer
+            if isinstance(m, LatentAttentionSpec):
+                n += 3 * d + m.q_rank * (d + 1) + m.heads * (m.dim + m.rot_dim) * m.q_rank \
+                    + m.heads * (m.dim + m.vdim) * m.kv_rank + m.gate_rows * d \
+                    + d * m.heads * m.vdim
+                if m.kv_from is None:
+                    n += m.cache_dim * d + m.kv_rank
+                if ls.mlp is not None:
+                    e = ls.mlp.router.experts if ls.mlp.router else 1
+                    n += 2 * d * ls.mlp.ff * e
+                    if ls.mlp.router:
+                        n += ls.mlp.router.outputs * (d + 1)
+                continue
             n += d + (m.heads + m.kv_heads) * m.dim * (d + 2) + m.heads * (d + 1) \
                 + d * (m.heads * m.vdim + 1)
             if ls.mlp is not None:
@@ -222,8 +294,98 @@ def bidetar_config(name: str, d: dict, max_position: int = 1 << 20) -> LayeredCo
     return cfg
 
 
+def _puputar_layer(ly: dict) -> LayerSpec:
+    kinds = {"latent_attention": "head", "latent_attention_2": "element"}
+    if ly["type"] not in kinds:
+        raise ValueError(f"Puputar: unknown mixer type {ly['type']!r}")
+    m = ly["mixer"]
+    rot = m["rot"]
+    if int(rot["dims"]) != int(m["rot_dim"]) or int(m["rot_dim"]) % 2:
+        raise ValueError("Puputar: the rotated part is rotated whole (rot.dims == rot_dim, even)")
+    kv_from = m.get("kv_from")
+    mixer = LatentAttentionSpec(
+        heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+        kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]), scale=float(m["scale"]),
+        rot=RotarySpec(int(rot["dims"]), float(rot["base"])), gate=kinds[ly["type"]],
+        kv_from=None if kv_from is None else int(kv_from))
+    ml = ly.get("mlp")
+    mlp = None
+    if ml is not None:
+        if ml["kind"] == "dense":
+            mlp = MlpSpec("dense", int(ml["ff"]), act="xielu", bias=True)
+        elif ml["kind"] == "moe":
+            rt, gr = ml["router"], ml["router"].get("groups") or {}
+            router = RouterSpec(experts=int(rt["experts"]), top=int(rt["top"]),
+                                identity=int(rt.get("identity") or 0),
+                                groups=int(gr.get("count") or 1), keep=int(gr.get("keep") or 1))
+            if router.outputs % router.groups or not 1 <= router.keep <= router.groups \
+                    or router.top > router.keep * (router.outputs // router.groups):
+                raise ValueError(f"Puputar: bad router {rt}")
+            mlp = MlpSpec("moe", int(ml["expert"]["ff"]), act="relu2", router=router)
+        else:
+            raise ValueError(f"Puputar: unknown feed-forward kind {ml['kind']!r}")
+    return LayerSpec(ly["type"], mixer, mlp)
+
+
+def puputar_config(name: str, d: dict, max_position: int = 1 << 20) -> LayeredConfig:
+    """A Puputar config.json: parallel layers with two grouped RMS norms (one feeds the mixer
+    through a token shift, one the feed-forward), latent attention mixers (per-head or
+    per-element output gate, optionally reading an earlier layer's cached latent) and dense
+    xIELU or routed squared-ReLU feed-forwards."""
+    specs = [_puputar_layer(ly) for ly in d["layers"]]
+    for i, ls in enumerate(specs):
+        j = ls.mixer.kv_from
+        if j is None:
+            continue
+        if not 0 <= j < i or specs[j].mixer.kv_from is not None:
+            raise ValueError(f"Puputar: layer {i} reads the cache of layer {j}, which must be an "
+                             "earlier layer with a cache of its own")
+        a, b = ls.mixer, specs[j].mixer
+        if (a.kv_rank, a.rot_dim, a.rot.base) != (b.kv_rank, b.rot_dim, b.rot.base):
+            raise ValueError(f"Puputar: layers {i} and {j} share a cache of unequal shape")
+    width, groups = int(d["width"]), int(d["norm"].get("groups") or 1)
+    if width % groups:
+        raise ValueError("Puputar: width must be a multiple of norm.groups")
+    cfg = LayeredConfig(
+        name=name, hf_id=name, arch="puputar", vocab_size=int(d["vocab"]), hidden_size=width,
+        intermediate_size=max([ls.mlp.ff for ls in specs if ls.mlp is not None] or [0]),
+        num_layers=len(specs), num_heads=max(ls.mixer.heads for ls in specs), num_kv_heads=1,
+        head_dim=max(ls.mixer.cache_dim for ls in specs), rms_eps=float(d["norm"]["eps"]),
+        max_position=max_position, bos_id=0, eos_id=-1, layer_specs=specs, norm_groups=groups)
+    return cfg
+
+
+def puputar_dict(width: int, layers: list, vocab: int = 32000, eps: float = 1e-6,
+                 norm_groups: int = 1) -> dict:
+    """A Puputar config.json dictionary from short layer tuples (random-init benchmarks and
+    tests): each layer is a dict with heads, dim, rot_dim, vdim, kv_rank, q_rank and optional
+    base, scale, gate ("head" | "element"), kv_from, and ff (dense), or experts / expert_ff /
+    top / identity / groups / keep (routed), or neither (no feed-forward)."""
+    out = []
+    for ly in layers:
+        m = {"heads": ly["heads"], "dim": ly["dim"], "rot_dim": ly["rot_dim"], "vdim": ly["vdim"],
+             "kv_rank": ly["kv_rank"], "q_rank": ly["q_rank"],
+             "rot": {"base": float(ly.get("base", 10000.0)), "dims": ly["rot_dim"]},
+             "scale": float(ly.get("scale", (ly["dim"] + ly["rot_dim"]) ** -0.5))}
+        if ly.get("kv_from") is not None:
+            m["kv_from"] = ly["kv_from"]
+        if "experts" in ly:
+            mlp = {"kind": "moe", "expert": {"ff": ly["expert_ff"]},
+                   "router": {"experts": ly["experts"], "top": ly["top"],
+                              "identity": ly.get("identity", 0),
+                              "groups": {"count": ly.get("groups", 1), "keep": ly.get("keep", 1)}}}
+        elif ly.get("ff"):
+            mlp = {"kind": "dense", "ff": ly["ff"]}
+        else:
+            mlp = None
+        out.append({"type": "latent_attention_2" if ly.get("gate") == "element"
+                    else "latent_attention", "mixer": m, "mlp": mlp})
+    return {"architecture": "Puputar", "layers": out, "norm": {"eps": eps, "groups": norm_groups},
+            "vocab": vocab, "width": width}
+
+
 # config.json readers of designs that do not use the HF key set, by their "architecture" value
-_NATIVE_READERS = {"Bidetar": bidetar_config}
+_NATIVE_READERS = {"Bidetar": bidetar_config, "Puputar": puputar_config}
 
 _REGISTRY: dict[str, ModelConfig] = {}
 
@@ -363,6 +525,47 @@ BIDETAR_W1536 = register(layered_config(
 TINY_BIDETAR = register(layered_config(
     "tiny-bidetar", width=128, num_layers=3, heads=4, kv_heads=2, dim=32, ff=256, chunk=48,
     vocab=512, loop=(1, 3, 2), rot_dims=16, residual_mult=0.7, embed_scale=4.0))
+
+
+def _puputar_stack(name: str, width: int, n: int, heads: int, dim: int, rot_dim: int, vdim: int,
+                   kv_rank: int, q_rank: int, ff: int, experts: int = 0, expert_ff: int = 0,
+                   top: int = 0, identity: int = 0, groups: int = 1, keep: int = 1,
+                   vocab: int = 32000, norm_groups: int = 1) -> LayeredConfig:
+    """n layers; every second one after the first has a routed feed-forward (when experts > 0),
+    every third gates per element, and the last of those reads the first one's cache."""
+    layers, first_el = [], None
+    for i in range(n):
+        ly = dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank,
+                  q_rank=q_rank)
+        if i % 3 == 1:
+            ly["gate"] = "element"
+            if first_el is None:
+                first_el = i
+            elif i + 3 >= n:
+                ly["kv_from"] = first_el
+        if experts and i and i % 2 == 0:
+            ly.update(experts=experts, expert_ff=expert_ff, top=top, identity=identity,
+                      groups=groups, keep=keep)
+        else:
+            ly["ff"] = ff
+        layers.append(ly)
+    cfg = puputar_config(name, puputar_dict(width, layers, vocab=vocab, norm_groups=norm_groups))
+    cfg.hf_id = "test/" + name
+    return cfg
+
+
+# Puputar at layer sizes of real models (random weights; bench.py --compare-design puputar):
+# 128 + 64 query/key dimensions per head over a 512 + 64 latent cache
+PUPUTAR_W2048 = register(_puputar_stack(
+    "puputar-w2048", width=2048, n=16, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512,
+    q_rank=768, ff=8192))
+PUPUTAR_W2048_MOE = register(_puputar_stack(
+    "puputar-w2048-moe", width=2048, n=16, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512,
+    q_rank=768, ff=8192, experts=14, expert_ff=2048, top=4, identity=2, groups=4, keep=2))
+TINY_PUPUTAR = register(_puputar_stack(
+    "tiny-puputar", width=128, n=6, heads=4, dim=16, rot_dim=8, vdim=24, kv_rank=40, q_rank=48,
+    ff=192, experts=6, expert_ff=64, top=3, identity=2, groups=4, keep=2, vocab=512,
+    norm_groups=4))
 
 
 def get_config(name: str) -> ModelConfig:

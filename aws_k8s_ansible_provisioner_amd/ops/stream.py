@@ -289,3 +289,253 @@ def sink_attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Ten
             _attend_rows(out, q, k_cache, v_cache, block_tables[b], kv, kv - 1, slice(b, b + 1),
                          gate, sink, scale, chunk, window)
     return out
+
+
+# ----------------------------------------------------------------------------- grouped norms
+def _group_rms(x: torch.Tensor, groups: int, eps: float) -> torch.Tensor:
+    T, d = x.shape
+    return _rms(x.view(T, groups, d // groups), eps).view(T, d)
+
+
+def stream_add_group_norm(x: torch.Tensor, y: Optional[torch.Tensor], y2: Optional[torch.Tensor],
+                          bias: Optional[torch.Tensor], w1: torch.Tensor,
+                          w2: Optional[torch.Tensor], groups: int, eps: float,
+                          out1: torch.Tensor, out2: Optional[torch.Tensor] = None) -> None:
+    """x += y + bias + y2 in place (fp32 stream; y [T, d] and bias [d] in the activation type,
+    y2 [T, d] fp32; each may be None), then the RMS norm of the new x in `groups` equal
+    consecutive parts (each divided by its own root mean square), written twice: out1 with the
+    weights w1 and out2 with w2 (None: one output).  One pass over the row serves the residual
+    update and both norms of a layer whose mixer and feed-forward read differently-weighted
+    norms of the same stream."""
+    if _native(x):
+        torch.ops.akap_stream.add_group_norm(out1, out2, x, y, y2, bias, w1, w2, int(groups),
+                                             float(eps))
+        return
+    if y is not None:
+        x.add_(y.float())
+    if bias is not None:
+        x.add_(bias.float())
+    if y2 is not None:
+        x.add_(y2)
+    n = _group_rms(x, groups, eps)
+    out1.copy_((n * w1.float()).to(out1.dtype))
+    if out2 is not None:
+        out2.copy_((n * w2.float()).to(out2.dtype))
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, seq_slot: torch.Tensor,
+                positions: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t] = h[t] + (prev_t - h[t]) * mu, where prev_t is the UNSHIFTED row of the token
+    before t in its sequence: row t-1 when that row is the same sequence's previous position
+    (equal seq_slot, positions[t-1] + 1 == positions[t]), zeros at position 0, else what an
+    earlier step left in state[seq_slot[t]].  Then state[seq_slot[t]] = h[t] for the last row of
+    every sequence in the batch.  state [slots, d] (h's type), mu [d] fp32, seq_slot int32
+    (-1: a padding row, no state read or written)."""
+    if _native(h):
+        torch.ops.akap_stream.token_shift(out, h, mu, state, seq_slot, positions)
+        return
+    T = h.shape[0]
+    slot, pos = seq_slot.long(), positions.long()
+    cont = torch.zeros(T, dtype=torch.bool)
+    cont[1:] = (slot[1:] == slot[:-1]) & (pos[1:] == pos[:-1] + 1) & (slot[1:] >= 0)
+    prev = torch.zeros(T, h.shape[1], dtype=torch.float32)
+    prev[1:][cont[1:]] = h[:-1][cont[1:]].float()
+    old = ~cont & (pos > 0) & (slot >= 0)
+    prev[old] = state[slot[old]].float()
+    last = torch.ones(T, dtype=torch.bool)
+    last[:-1] = ~cont[1:]
+    last &= slot >= 0
+    hf = h.float()
+    new_state = h[last].clone()
+    out.copy_((hf + (prev - hf) * mu.float()).to(out.dtype))
+    state[slot[last]] = new_state
+
+
+# ----------------------------------------------------------------------------- latent attention
+def _rotate_pairs(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
+    """x [T, ..., dims] rotated in interleaved pairs by the table rows cs [T, dims]."""
+    dims = cs.shape[1]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [dims // 2]
+    c, s = cs[:, :dims // 2].reshape(shape), cs[:, dims // 2:].reshape(shape)
+    u, v = x[..., 0::2], x[..., 1::2]
+    o = torch.empty_like(x)
+    o[..., 0::2] = u * c - v * s
+    o[..., 1::2] = v * c + u * s
+    return o
+
+
+def latent_prep(proj: torch.Tensor, cq_out: torch.Tensor, cache: Optional[torch.Tensor],
+                positions: torch.Tensor, slots: torch.Tensor, cos_sin: torch.Tensor,
+                q_w: torch.Tensor, kv_w: Optional[torch.Tensor], q_rank: int, kv_rank: int,
+                rot_dim: int, q_off: int, kv_off: int, eps: float) -> None:
+    """Per token t of the fused down-projection proj [T, N]: the query latent
+    proj[t, q_off : q_off + q_rank] is RMS-normalised (weights q_w, fp32) into cq_out
+    [T, q_rank]; the key/value latent proj[t, kv_off : kv_off + kv_rank] is RMS-normalised
+    (kv_w) and the next rot_dim entries rotated in interleaved pairs by the angle row of
+    positions[t], and both are written as one row [kv_rank + rot_dim] of the paged latent
+    cache [NB, BS, kv_rank + rot_dim] at slots[t] (-1: nothing).  cache None: the layer reads
+    another layer's cache and projects no latent of its own."""
+    if _native(proj):
+        torch.ops.akap_stream.latent_prep(proj, cq_out, cache, positions, slots, cos_sin, q_w,
+                                          kv_w, q_rank, kv_rank, rot_dim, q_off, kv_off,
+                                          float(eps))
+        return
+    cq = _rms(proj[:, q_off:q_off + q_rank].float(), eps) * q_w.float()
+    cq_out.copy_(cq.to(cq_out.dtype))
+    if cache is None:
+        return
+    c = _rms(proj[:, kv_off:kv_off + kv_rank].float(), eps) * kv_w.float()
+    kr = _rotate_pairs(proj[:, kv_off + kv_rank:kv_off + kv_rank + rot_dim].float(),
+                       cos_sin[positions.long()])
+    BS = cache.shape[1]
+    ok = slots >= 0
+    sl = slots[ok].long()
+    cache[sl // BS, sl % BS] = torch.cat([c, kr], dim=1)[ok].to(cache.dtype)
+
+
+def rotate_heads_(q: torch.Tensor, positions: torch.Tensor, cos_sin: torch.Tensor,
+                  offset: int) -> None:
+    """In place: the cos_sin.shape[1] entries from `offset` of every head of q [T, H, n] are
+    rotated in interleaved pairs by the angle row of positions[t] (fp32 arithmetic)."""
+    if _native(q):
+        torch.ops.akap_stream.rotate_heads(q, positions, cos_sin, int(offset))
+        return
+    dims = cos_sin.shape[1]
+    part = q[:, :, offset:offset + dims].float()
+    q[:, :, offset:offset + dims] = _rotate_pairs(part, cos_sin[positions.long()]).to(q.dtype)
+
+
+def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q: torch.Tensor, rot_off: int,
+                     cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
+                     q_start: Optional[torch.Tensor], positions: torch.Tensor,
+                     scale: float) -> None:
+    """Causal softmax attention of every head against ONE cached row per key: the score of
+    query (t, h) and key j is (q_lat[h, t] . cache[j, :R] + q[t, h, rot_off:rot_off + r] .
+    cache[j, R:R + r]) * scale, where q_lat [H, T, R] is the unrotated query already multiplied
+    into the latent space (W_uk^T q), and out[h, t] = sum_j softmax_j(score) cache[j, :R]
+    (still latent: the caller applies W_uv per head).  The keys of token t are positions
+    0 .. positions[t] of its sequence's block-table row; its sequence is b with
+    q_start[b] <= t < q_start[b+1] (q_start None: row t is sequence t, one query each).
+    Sequences with seq_lens[b] == 0 are padding.  Scores and softmax are fp32."""
+    if _native(q):
+        torch.ops.akap_stream.latent_attention(out, q_lat, q, int(rot_off), cache, block_tables,
+                                               seq_lens, q_start, positions, float(scale))
+        return
+    H, T, R = q_lat.shape
+    BS, r = cache.shape[1], cache.shape[2] - R
+    B = seq_lens.numel()
+    for b in range(B):
+        kv = int(seq_lens[b])
+        if kv == 0:
+            continue
+        r0, r1 = (b, b + 1) if q_start is None else (int(q_start[b]), int(q_start[b + 1]))
+        if r1 <= r0:
+            continue
+        nb = -(-kv // BS)
+        rows = cache[block_tables[b, :nb].long()].reshape(nb * BS, R + r)[:kv].float()
+        pos = positions[r0:r1].long()
+        ok = torch.arange(kv)[None, :] <= pos[:, None]
+        s = torch.einsum("htr,jr->htj", q_lat[:, r0:r1].float(), rows[:, :R]) + \
+            torch.einsum("thr,jr->htj", q[r0:r1, :, rot_off:rot_off + r].float(), rows[:, R:])
+        s = (s * scale).masked_fill(~ok[None], float("-inf"))
+        out[:, r0:r1] = torch.einsum("htj,jr->htr", torch.softmax(s, dim=-1),
+                                     rows[:, :R]).to(out.dtype)
+
+
+def head_gate(o: torch.Tensor, gate: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, h V + j] = o[h, t, j] * sigmoid(g), g = gate[t, h] when gate has H columns (one
+    gate per head) or gate[t, h V + j] when it has H V (one per output entry).  o [H, T, V]
+    (head-major, as the per-head up-projection leaves it), gate and out are [T, .] views that
+    may be column slices of wider rows.  The sigmoid and the product are fp32."""
+    if _native(o):
+        torch.ops.akap_stream.head_gate(out, o, gate)
+        return
+    H, T, V = o.shape
+    g = torch.sigmoid(gate.float())
+    g = g[:, :, None] if gate.shape[1] == H else g.view(T, H, V)
+    out.copy_((o.float().permute(1, 0, 2) * g).reshape(T, H * V).to(out.dtype))
+
+
+def xielu(x: torch.Tensor, bias: Optional[torch.Tensor], act: torch.Tensor,
+          out: torch.Tensor) -> None:
+    """out = f(x + bias), f(z) = softplus(p) z^2 + z / 2 for z > 0 and
+    (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2 otherwise, (p, q) = act (fp32 [2], read on
+    the device).  x and out are [T, F] views that may be column slices of wider rows."""
+    if _native(x):
+        torch.ops.akap_stream.xielu(out, x, bias, act)
+        return
+    z = x.float()
+    if bias is not None:
+        z = z + bias.float()
+    ap, aq = torch.nn.functional.softplus(act.float()[0]), torch.nn.functional.softplus(act.float()[1])
+    neg = torch.clamp(z, max=0.0)
+    out.copy_(torch.where(z > 0, ap * z * z + z / 2,
+                          (0.5 + aq) * (torch.expm1(neg) - neg) + z / 2).to(out.dtype))
+
+
+# ----------------------------------------------------------------------------- routed experts
+def moe_route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor],
+              top: int, groups: int = 1, keep: int = 1):
+    """Grouped top-k routing: scores s = softmax(router h) over all n router outputs (fp32
+    logits from h's stored values); the choice uses s + correction; outputs form `groups` equal
+    groups of neighbours, a group scores its largest choice value, and only outputs of the
+    `keep` best groups can be chosen; the `top` largest allowed choice values win (ties: the
+    lower index).  Returns ids int32 [T, top] and weights fp32 [T, top] = the winners' s
+    divided by their sum (+ 1e-20).  router fp32 [n, d], correction fp32 [n]."""
+    T, n = h.shape[0], router.shape[0]
+    ids = torch.empty(T, top, dtype=torch.int32, device=h.device)
+    w = torch.empty(T, top, dtype=torch.float32, device=h.device)
+    if _native(h):
+        torch.ops.akap_stream.moe_route(ids, w, h, router, correction, int(groups), int(keep))
+        return ids, w
+    s = torch.softmax(h.float() @ router.float().T, dim=-1)
+    choice = s + correction.float() if correction is not None else s.clone()
+    per = n // groups
+    if groups > 1:
+        gs = choice.view(T, groups, per).max(dim=-1).values
+        best = gs.topk(keep, dim=-1).indices
+        allowed = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, best, True)
+        choice = choice.masked_fill(~allowed[:, :, None].expand(T, groups, per).reshape(T, n),
+                                    float("-inf"))
+    idx = choice.topk(top, dim=-1).indices
+    sel = s.gather(1, idx)
+    ids.copy_(idx)
+    w.copy_(sel / (sel.sum(dim=-1, keepdim=True) + 1e-20))
+    return ids, w
+
+
+def relu2_routed(up: torch.Tensor, ids: torch.Tensor, w: torch.Tensor, experts: int,
+                 out: torch.Tensor) -> None:
+    """out[t, e F + f] = w_e(t) relu(up[t, e F + f])^2, w_e(t) the routing weight of expert e for
+    token t (0 when it was not chosen): the activation of EVERY expert's up-projection scaled so
+    that one GEMM with the concatenated down-projections [d, E F] sums the chosen experts
+    (small batches, where all expert weights are streamed anyway).  ids [T, top] >= experts are
+    identity outputs and scale nothing here."""
+    if _native(up):
+        torch.ops.akap_stream.relu2_routed(out, up, ids, w, int(experts))
+        return
+    T = up.shape[0]
+    F_ = up.shape[1] // experts
+    full = torch.zeros(T, experts + 1, dtype=torch.float32)
+    full.scatter_(1, ids.long().clamp(max=experts), w)
+    r = torch.relu(up.float()).view(T, experts, F_)
+    out.copy_((r * r * full[:, :experts, None]).view(T, experts * F_).to(out.dtype))
+
+
+def moe_combine(out: torch.Tensor, y: torch.Tensor, inv: Optional[torch.Tensor],
+                ids: torch.Tensor, w: torch.Tensor, h: torch.Tensor, experts: int) -> None:
+    """out (fp32 [T, d]) = the routed feed-forward's output.  inv None: y [T, d] already holds
+    the weighted sum over the chosen experts.  inv int32 [T, top]: y [T top, d] are expert
+    outputs in expert-sorted row order, inv[t, k] the row of choice k of token t, and
+    out[t] = sum_k w[t, k] y[inv[t, k]].  Either way choices with ids >= experts (identity
+    outputs) add w[t, k] h[t]."""
+    if _native(y):
+        torch.ops.akap_stream.moe_combine(out, y, inv, ids, w, h, int(experts))
+        return
+    ident = (w * (ids >= experts)).sum(dim=1, keepdim=True)
+    if inv is None:
+        acc = y.float()
+    else:
+        real = (w * (ids < experts))[:, :, None]
+        acc = (y.float()[inv.long().clamp(min=0, max=y.shape[0] - 1)] * real).sum(dim=1)
+    out.copy_(acc + ident * h.float())
