@@ -67,4 +67,69 @@ struct AttnParams {
 void launch_sink_attention_prefill(const AttnParams& p, bool f32, hipStream_t s);
 void launch_sink_attention_decode(const AttnParams& p, bool f32, hipStream_t s);
 
+// ---- grouped norms, token shift, latent attention, routed experts (latent.hip) ----------------
+// x (fp32 rows of d) += y + bias + y2 (each may be null; y / bias of the activation type, y2
+// fp32), then out1 = gnorm(x) * w1 and out2 = gnorm(x) * w2 (out2 / w2 may be null), the norm
+// taken over `groups` equal consecutive parts of the row
+void launch_add_group_norm(void* out1, void* out2, bool out_f32, int out1_stride, int out2_stride,
+                           float* x, const void* y, bool y_f32, int y_stride, const float* y2,
+                           const void* bias, const float* w1, const float* w2, int rows, int d,
+                           int groups, float eps, hipStream_t s);
+// out[t] = h[t] + (prev - h[t]) * mu; then the last row of each sequence goes to state[slot]
+void launch_token_shift(void* out, const void* h, const float* mu, void* state,
+                        const int32_t* slot, const int64_t* pos, bool f32, int rows, int d,
+                        hipStream_t s);
+
+struct LatentPrepParams {
+  const void* proj;   // [T, N] fused down-projection rows
+  int proj_stride;
+  void* cq_out;       // [T, q_rank]
+  void* cache;        // [NB * BS, kv_rank + rot_dim] or null
+  const int64_t* positions;
+  const int64_t* slots;
+  const float* cos_sin;  // [max_pos, rot_dim] = [cos | sin]
+  int max_pos;
+  const float* q_w;      // [q_rank]
+  const float* kv_w;     // [kv_rank]
+  int T, q_rank, kv_rank, rot_dim, q_off, kv_off;
+  int64_t num_slots;
+  float eps;
+};
+void launch_latent_prep(const LatentPrepParams& p, bool f32, hipStream_t s);
+// in place: `dims` entries from `offset` of each of the H heads (n entries per head) of a row
+void launch_rotate_heads(void* q, int q_stride, int T, int H, int n, int offset, int dims,
+                         const int64_t* positions, const float* cos_sin, int max_pos, bool f32,
+                         hipStream_t s);
+
+struct LatentAttnParams {
+  void* out;            // [H, T, R]
+  const void* q_lat;    // [H, T, R]
+  const void* q;        // [T, H, q_head]; the rotated part at rot_off of every head
+  int q_stride, q_head, rot_off;
+  const void* cache;    // [NB * BS, R + r]
+  const int32_t* block_tables;  // [B, max_blocks]
+  int max_blocks;
+  const int32_t* seq_lens;      // [B]
+  const int32_t* q_start;       // [B + 1], or null: row t is sequence t
+  const int64_t* positions;     // [T]
+  float scale;
+  int T, B, H, R, r, BS;
+  int vec;              // rows of the cache can be read in 16-byte pieces
+};
+void launch_latent_attention(const LatentAttnParams& p, bool f32, hipStream_t s);
+
+void launch_head_gate(void* out, int out_stride, const void* o, const void* gate, int gate_stride,
+                      bool per_head, int rows, int H, int V, bool f32, hipStream_t s);
+void launch_xielu(void* out, int out_stride, const void* x, int x_stride, const void* bias,
+                  const float* act, int rows, int F, bool f32, hipStream_t s);
+void launch_moe_route(int32_t* ids, float* w, const void* h, int h_stride, const float* router,
+                      const float* corr, int rows, int d, int n, int top, int groups, int keep,
+                      bool f32, hipStream_t s);
+void launch_relu2_routed(void* out, int out_stride, const void* up, int up_stride,
+                         const int32_t* ids, const float* w, int rows, int top, int E, int F,
+                         bool f32, hipStream_t s);
+void launch_moe_combine(float* out, const void* y, const int32_t* inv, const int32_t* ids,
+                        const float* w, const void* h, int h_stride, int rows, int d, int top,
+                        int E, int y_rows, bool f32, hipStream_t s);
+
 }  // namespace akap_stream

@@ -247,6 +247,304 @@ void sink_attention_decode(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
   akap_stream::launch_sink_attention_decode(p, is_f32(q, "q"), cur_stream());
 }
 
+
+// ---- grouped norms, token shift, latent attention, routed experts ----------------------------
+void add_group_norm(Tensor out1, std::optional<Tensor> out2, Tensor x, std::optional<Tensor> y,
+                    std::optional<Tensor> y2, std::optional<Tensor> bias, Tensor w1,
+                    std::optional<Tensor> w2, int64_t groups, double eps) {
+  CHECK_GPU(out1); CHECK_GPU(x); CHECK_GPU(w1);
+  CHECK_F32(x); CHECK_CONTIG(x); CHECK_F32(w1); CHECK_CONTIG(w1); CHECK_LAST_CONTIG(out1);
+  TORCH_CHECK(x.dim() == 2 && out1.dim() == 2 && out1.sizes() == x.sizes(),
+              "add_group_norm: shapes");
+  const int rows = x.size(0), d = x.size(1);
+  TORCH_CHECK(groups >= 1 && d % groups == 0, "add_group_norm: d must split into the groups");
+  TORCH_CHECK(w1.numel() == d, "add_group_norm: weight size");
+  TORCH_CHECK(out1.data_ptr() != x.data_ptr(), "add_group_norm: out1 must not alias x");
+  const bool of = is_f32(out1, "out1");
+  void* o2 = nullptr;
+  const float* w2p = nullptr;
+  int o2s = 0;
+  if (out2.has_value()) {
+    TORCH_CHECK(w2.has_value(), "add_group_norm: out2 needs w2");
+    CHECK_GPU(*out2); CHECK_LAST_CONTIG(*out2); CHECK_GPU(*w2); CHECK_F32(*w2); CHECK_CONTIG(*w2);
+    TORCH_CHECK(out2->sizes() == x.sizes() && out2->scalar_type() == out1.scalar_type() &&
+                    w2->numel() == d, "add_group_norm: out2 / w2");
+    o2 = out2->data_ptr();
+    o2s = out2->stride(0);
+    w2p = w2->data_ptr<float>();
+  }
+  const void* yp = nullptr;
+  bool yf = of;
+  int ys = 0;
+  if (y.has_value()) {
+    CHECK_GPU(*y); CHECK_LAST_CONTIG(*y);
+    TORCH_CHECK(y->dim() == 2 && y->sizes() == x.sizes(), "add_group_norm: y shape");
+    yp = y->data_ptr();
+    yf = is_f32(*y, "y");
+    ys = y->stride(0);
+  }
+  const void* bp = nullptr;
+  if (bias.has_value()) {
+    CHECK_GPU(*bias); CHECK_CONTIG(*bias);
+    TORCH_CHECK(bias->numel() == d, "add_group_norm: bias must be [d]");
+    if (y.has_value()) {
+      TORCH_CHECK(bias->scalar_type() == y->scalar_type(), "bias dtype != y dtype");
+    } else {
+      yf = is_f32(*bias, "bias");
+    }
+    bp = bias->data_ptr();
+  }
+  const float* y2p = nullptr;
+  if (y2.has_value()) {
+    CHECK_GPU(*y2); CHECK_F32(*y2); CHECK_CONTIG(*y2);
+    TORCH_CHECK(y2->sizes() == x.sizes(), "add_group_norm: y2 shape");
+    y2p = y2->data_ptr<float>();
+  }
+  const c10::DeviceGuard g(x.device());
+  akap_stream::launch_add_group_norm(out1.data_ptr(), o2, of, (int)out1.stride(0), o2s,
+                                     x.data_ptr<float>(), yp, yf, ys, y2p, bp,
+                                     w1.data_ptr<float>(), w2p, rows, d, (int)groups, (float)eps,
+                                     cur_stream());
+}
+
+void token_shift(Tensor out, Tensor h, Tensor mu, Tensor state, Tensor seq_slot, Tensor positions) {
+  CHECK_GPU(out); CHECK_GPU(h); CHECK_GPU(mu); CHECK_GPU(state); CHECK_GPU(seq_slot);
+  CHECK_GPU(positions);
+  CHECK_CONTIG(out); CHECK_CONTIG(h); CHECK_CONTIG(mu); CHECK_CONTIG(state); CHECK_CONTIG(seq_slot);
+  CHECK_CONTIG(positions); CHECK_F32(mu);
+  TORCH_CHECK(h.dim() == 2 && out.sizes() == h.sizes() && state.dim() == 2, "token_shift: shapes");
+  const int64_t T = h.size(0), d = h.size(1);
+  TORCH_CHECK(out.scalar_type() == h.scalar_type() && state.scalar_type() == h.scalar_type(),
+              "token_shift: dtypes differ");
+  TORCH_CHECK(out.data_ptr() != h.data_ptr(), "token_shift: out must not alias h");
+  TORCH_CHECK(mu.numel() == d && state.size(1) == d, "token_shift: width");
+  TORCH_CHECK(seq_slot.scalar_type() == at::kInt && positions.scalar_type() == at::kLong,
+              "token_shift: seq_slot int32, positions int64");
+  TORCH_CHECK(seq_slot.numel() >= T && positions.numel() >= T, "token_shift: per-row inputs");
+  // slots index state rows: checked on the host side of the scheduler (slots < pool size)
+  const c10::DeviceGuard g(h.device());
+  akap_stream::launch_token_shift(out.data_ptr(), h.data_ptr(), mu.data_ptr<float>(),
+                                  state.data_ptr(), seq_slot.data_ptr<int32_t>(),
+                                  positions.data_ptr<int64_t>(), is_f32(h, "h"), (int)T, (int)d,
+                                  cur_stream());
+}
+
+void latent_prep(Tensor proj, Tensor cq_out, std::optional<Tensor> cache, Tensor positions,
+                 Tensor slots, Tensor cos_sin, Tensor q_w, std::optional<Tensor> kv_w,
+                 int64_t q_rank, int64_t kv_rank, int64_t rot_dim, int64_t q_off, int64_t kv_off,
+                 double eps) {
+  CHECK_GPU(proj); CHECK_LAST_CONTIG(proj); CHECK_GPU(cq_out); CHECK_CONTIG(cq_out);
+  CHECK_GPU(positions); CHECK_GPU(slots); CHECK_CONTIG(positions); CHECK_CONTIG(slots);
+  CHECK_GPU(cos_sin); CHECK_F32(cos_sin); CHECK_CONTIG(cos_sin);
+  CHECK_GPU(q_w); CHECK_F32(q_w); CHECK_CONTIG(q_w);
+  TORCH_CHECK(positions.scalar_type() == at::kLong && slots.scalar_type() == at::kLong,
+              "positions/slots must be int64");
+  const bool f32 = is_f32(proj, "proj");
+  TORCH_CHECK(proj.dim() == 2 && cq_out.scalar_type() == proj.scalar_type(), "latent_prep: proj");
+  const int64_t T = proj.size(0);
+  TORCH_CHECK(q_rank > 0 && q_off >= 0 && q_off + q_rank <= proj.size(1), "q slice");
+  TORCH_CHECK(cq_out.numel() == T * q_rank && q_w.numel() == q_rank, "cq_out / q_w size");
+  TORCH_CHECK(positions.numel() >= T && slots.numel() >= T, "positions/slots too short");
+  akap_stream::LatentPrepParams p{};
+  p.proj = proj.data_ptr();
+  p.proj_stride = proj.stride(0);
+  p.cq_out = cq_out.data_ptr();
+  p.positions = positions.data_ptr<int64_t>();
+  p.slots = slots.data_ptr<int64_t>();
+  p.cos_sin = cos_sin.data_ptr<float>();
+  p.max_pos = cos_sin.size(0);
+  p.q_w = q_w.data_ptr<float>();
+  p.T = T; p.q_rank = q_rank; p.kv_rank = kv_rank; p.rot_dim = rot_dim; p.q_off = q_off;
+  p.kv_off = kv_off;
+  p.eps = (float)eps;
+  if (cache.has_value()) {
+    CHECK_GPU(*cache); CHECK_CONTIG(*cache);
+    TORCH_CHECK(kv_w.has_value(), "latent_prep: a cache needs kv_w");
+    CHECK_GPU(*kv_w); CHECK_F32(*kv_w); CHECK_CONTIG(*kv_w);
+    TORCH_CHECK(cache->dim() == 3 && cache->size(2) == kv_rank + rot_dim &&
+                    cache->scalar_type() == proj.scalar_type(), "latent cache [NB, BS, R + r]");
+    TORCH_CHECK(kv_rank > 0 && rot_dim > 0 && rot_dim % 2 == 0 && kv_off >= 0 &&
+                    kv_off + kv_rank + rot_dim <= proj.size(1), "kv slice");
+    TORCH_CHECK(kv_w->numel() == kv_rank && cos_sin.dim() == 2 && cos_sin.size(1) == rot_dim,
+                "kv_w / rotary table size");
+    p.cache = cache->data_ptr();
+    p.kv_w = kv_w->data_ptr<float>();
+    p.num_slots = cache->size(0) * cache->size(1);
+  }
+  const c10::DeviceGuard g(proj.device());
+  akap_stream::launch_latent_prep(p, f32, cur_stream());
+}
+
+void rotate_heads(Tensor q, Tensor positions, Tensor cos_sin, int64_t offset) {
+  CHECK_GPU(q); CHECK_GPU(positions); CHECK_GPU(cos_sin); CHECK_F32(cos_sin); CHECK_CONTIG(cos_sin);
+  CHECK_CONTIG(positions);
+  TORCH_CHECK(q.dim() == 3 && q.stride(2) == 1 && q.stride(1) == q.size(2), "q must be [T, H, n]");
+  TORCH_CHECK(positions.scalar_type() == at::kLong && positions.numel() >= q.size(0), "positions");
+  const int64_t dims = cos_sin.size(1);
+  TORCH_CHECK(cos_sin.dim() == 2 && dims % 2 == 0 && offset >= 0 && offset + dims <= q.size(2),
+              "rotated part outside the head");
+  const c10::DeviceGuard g(q.device());
+  akap_stream::launch_rotate_heads(q.data_ptr(), (int)q.stride(0), (int)q.size(0), (int)q.size(1),
+                                   (int)q.size(2), (int)offset, (int)dims,
+                                   positions.data_ptr<int64_t>(), cos_sin.data_ptr<float>(),
+                                   (int)cos_sin.size(0), is_f32(q, "q"), cur_stream());
+}
+
+void latent_attention(Tensor out, Tensor q_lat, Tensor q, int64_t rot_off, Tensor cache,
+                      Tensor block_tables, Tensor seq_lens, std::optional<Tensor> q_start,
+                      Tensor positions, double scale) {
+  CHECK_GPU(out); CHECK_GPU(q_lat); CHECK_GPU(q); CHECK_GPU(cache); CHECK_GPU(block_tables);
+  CHECK_GPU(seq_lens); CHECK_GPU(positions);
+  CHECK_CONTIG(out); CHECK_CONTIG(q_lat); CHECK_CONTIG(cache); CHECK_CONTIG(seq_lens);
+  CHECK_CONTIG(positions);
+  const bool f32 = is_f32(q, "q");
+  TORCH_CHECK(out.scalar_type() == q.scalar_type() && q_lat.scalar_type() == q.scalar_type() &&
+                  cache.scalar_type() == q.scalar_type(), "latent_attention: dtypes differ");
+  TORCH_CHECK(q_lat.dim() == 3 && out.sizes() == q_lat.sizes() && q.dim() == 3 &&
+                  q.stride(2) == 1 && q.stride(1) == q.size(2), "latent_attention: q shapes");
+  const int64_t H = q_lat.size(0), T = q_lat.size(1), R = q_lat.size(2);
+  TORCH_CHECK(q.size(0) == T && q.size(1) == H, "latent_attention: q is [T, H, n]");
+  TORCH_CHECK(cache.dim() == 3 && cache.size(2) > R, "latent cache [NB, BS, R + r]");
+  const int64_t r = cache.size(2) - R;
+  TORCH_CHECK(rot_off >= 0 && rot_off + r <= q.size(2), "rotated query part outside the head");
+  TORCH_CHECK(R <= 1024, "latent size over 1024");
+  TORCH_CHECK(block_tables.dim() == 2 && block_tables.scalar_type() == at::kInt &&
+                  block_tables.stride(1) == 1, "block_tables");
+  TORCH_CHECK(seq_lens.scalar_type() == at::kInt && positions.scalar_type() == at::kLong &&
+                  positions.numel() >= T, "seq_lens int32, positions int64");
+  const int64_t B = seq_lens.numel();
+  TORCH_CHECK(block_tables.size(0) >= B, "block table rows");
+  TORCH_CHECK(block_tables.size(1) * cache.size(1) < (1LL << 31), "sequence too long");
+  akap_stream::LatentAttnParams p{};
+  if (q_start.has_value()) {
+    CHECK_GPU(*q_start); CHECK_CONTIG(*q_start);
+    TORCH_CHECK(q_start->scalar_type() == at::kInt && q_start->numel() >= B + 1, "q_start");
+    p.q_start = q_start->data_ptr<int32_t>();
+  } else {
+    TORCH_CHECK(B >= T, "one query per sequence needs a sequence per row");
+  }
+  p.out = out.data_ptr();
+  p.q_lat = q_lat.data_ptr();
+  p.q = q.data_ptr();
+  p.q_stride = q.stride(0);
+  p.q_head = q.size(2);
+  p.rot_off = rot_off;
+  p.cache = cache.data_ptr();
+  p.block_tables = block_tables.data_ptr<int32_t>();
+  p.max_blocks = block_tables.stride(0);
+  p.seq_lens = seq_lens.data_ptr<int32_t>();
+  p.positions = positions.data_ptr<int64_t>();
+  p.scale = (float)scale;
+  p.T = T; p.B = B; p.H = H; p.R = R; p.r = r; p.BS = cache.size(1);
+  const int64_t es = f32 ? 4 : 2;
+  p.vec = ((R + r) * es) % 16 == 0 && ((uintptr_t)cache.data_ptr() % 16) == 0;
+  TORCH_CHECK(4 * (R + r) * 4 <= 64 * 1024, "query rows do not fit the LDS");
+  TORCH_CHECK((H + 3) / 4 <= 65535, "too many heads");
+  const c10::DeviceGuard g(q.device());
+  akap_stream::launch_latent_attention(p, f32, cur_stream());
+}
+
+void head_gate(Tensor out, Tensor o, Tensor gate) {
+  CHECK_GPU(out); CHECK_GPU(o); CHECK_GPU(gate); CHECK_CONTIG(o); CHECK_LAST_CONTIG(out);
+  CHECK_LAST_CONTIG(gate);
+  TORCH_CHECK(o.dim() == 3 && out.dim() == 2 && gate.dim() == 2, "head_gate: shapes");
+  const int64_t H = o.size(0), T = o.size(1), V = o.size(2);
+  TORCH_CHECK(out.size(0) == T && out.size(1) == H * V && gate.size(0) == T &&
+                  (gate.size(1) == H || gate.size(1) == H * V), "head_gate: sizes");
+  TORCH_CHECK(out.scalar_type() == o.scalar_type() && gate.scalar_type() == o.scalar_type(),
+              "head_gate: dtypes differ");
+  const c10::DeviceGuard g(o.device());
+  // H == H V only when V == 1: per-head and per-entry gates coincide
+  akap_stream::launch_head_gate(out.data_ptr(), (int)out.stride(0), o.data_ptr(), gate.data_ptr(),
+                                (int)gate.stride(0), gate.size(1) == H, (int)T, (int)H, (int)V,
+                                is_f32(o, "o"), cur_stream());
+}
+
+void xielu(Tensor out, Tensor x, std::optional<Tensor> bias, Tensor act) {
+  CHECK_GPU(out); CHECK_GPU(x); CHECK_GPU(act); CHECK_LAST_CONTIG(out); CHECK_LAST_CONTIG(x);
+  CHECK_F32(act); CHECK_CONTIG(act);
+  TORCH_CHECK(x.dim() == 2 && out.sizes() == x.sizes() && out.scalar_type() == x.scalar_type() &&
+                  act.numel() == 2, "xielu: shapes");
+  const void* bp = nullptr;
+  if (bias.has_value()) {
+    CHECK_GPU(*bias); CHECK_CONTIG(*bias);
+    TORCH_CHECK(bias->numel() == x.size(1) && bias->scalar_type() == x.scalar_type(), "xielu: bias");
+    bp = bias->data_ptr();
+  }
+  const c10::DeviceGuard g(x.device());
+  akap_stream::launch_xielu(out.data_ptr(), (int)out.stride(0), x.data_ptr(), (int)x.stride(0), bp,
+                            act.data_ptr<float>(), (int)x.size(0), (int)x.size(1), is_f32(x, "x"),
+                            cur_stream());
+}
+
+void moe_route(Tensor ids, Tensor w, Tensor h, Tensor router, std::optional<Tensor> correction,
+               int64_t groups, int64_t keep) {
+  CHECK_GPU(ids); CHECK_GPU(w); CHECK_GPU(h); CHECK_GPU(router);
+  CHECK_CONTIG(ids); CHECK_CONTIG(w); CHECK_LAST_CONTIG(h); CHECK_CONTIG(router);
+  CHECK_F32(w); CHECK_F32(router);
+  TORCH_CHECK(h.dim() == 2 && router.dim() == 2 && router.size(1) == h.size(1), "moe_route: width");
+  const int64_t T = h.size(0), n = router.size(0);
+  TORCH_CHECK(ids.scalar_type() == at::kInt && ids.dim() == 2 && ids.size(0) == T &&
+                  w.sizes() == ids.sizes(), "moe_route: ids / w [T, top]");
+  const int64_t top = ids.size(1);
+  TORCH_CHECK(groups >= 1 && n % groups == 0 && keep >= 1 && keep <= groups &&
+                  top >= 1 && top <= keep * (n / groups), "moe_route: groups / keep / top");
+  TORCH_CHECK((2 * n + groups) * 4 <= 48 * 1024, "moe_route: too many router outputs");
+  const float* cp = nullptr;
+  if (correction.has_value()) {
+    CHECK_GPU(*correction); CHECK_F32(*correction); CHECK_CONTIG(*correction);
+    TORCH_CHECK(correction->numel() == n, "moe_route: correction size");
+    cp = correction->data_ptr<float>();
+  }
+  const c10::DeviceGuard g(h.device());
+  akap_stream::launch_moe_route(ids.data_ptr<int32_t>(), w.data_ptr<float>(), h.data_ptr(),
+                                (int)h.stride(0), router.data_ptr<float>(), cp, (int)T,
+                                (int)h.size(1), (int)n, (int)top, (int)groups, (int)keep,
+                                is_f32(h, "h"), cur_stream());
+}
+
+void relu2_routed(Tensor out, Tensor up, Tensor ids, Tensor w, int64_t experts) {
+  CHECK_GPU(out); CHECK_GPU(up); CHECK_GPU(ids); CHECK_GPU(w);
+  CHECK_LAST_CONTIG(out); CHECK_LAST_CONTIG(up); CHECK_CONTIG(ids); CHECK_CONTIG(w); CHECK_F32(w);
+  TORCH_CHECK(up.dim() == 2 && out.sizes() == up.sizes() && out.scalar_type() == up.scalar_type(),
+              "relu2_routed: shapes");
+  TORCH_CHECK(experts >= 1 && up.size(1) % experts == 0 && experts * 4 <= 48 * 1024,
+              "relu2_routed: experts");
+  TORCH_CHECK(ids.scalar_type() == at::kInt && ids.dim() == 2 && ids.size(0) == up.size(0) &&
+                  w.sizes() == ids.sizes() && ids.size(1) <= 256, "relu2_routed: ids / w");
+  const c10::DeviceGuard g(up.device());
+  akap_stream::launch_relu2_routed(out.data_ptr(), (int)out.stride(0), up.data_ptr(),
+                                   (int)up.stride(0), ids.data_ptr<int32_t>(), w.data_ptr<float>(),
+                                   (int)up.size(0), (int)ids.size(1), (int)experts,
+                                   (int)(up.size(1) / experts), is_f32(up, "up"), cur_stream());
+}
+
+void moe_combine(Tensor out, Tensor y, std::optional<Tensor> inv, Tensor ids, Tensor w, Tensor h,
+                 int64_t experts) {
+  CHECK_GPU(out); CHECK_GPU(y); CHECK_GPU(ids); CHECK_GPU(w); CHECK_GPU(h);
+  CHECK_F32(out); CHECK_CONTIG(out); CHECK_CONTIG(y); CHECK_CONTIG(ids); CHECK_CONTIG(w);
+  CHECK_F32(w); CHECK_LAST_CONTIG(h);
+  TORCH_CHECK(out.dim() == 2 && h.dim() == 2 && h.sizes() == out.sizes() && y.dim() == 2 &&
+                  y.size(1) == out.size(1) && y.scalar_type() == h.scalar_type(),
+              "moe_combine: shapes");
+  const int64_t T = out.size(0);
+  TORCH_CHECK(ids.scalar_type() == at::kInt && ids.dim() == 2 && ids.size(0) == T &&
+                  w.sizes() == ids.sizes(), "moe_combine: ids / w");
+  const int32_t* ip = nullptr;
+  if (inv.has_value()) {
+    CHECK_GPU(*inv); CHECK_CONTIG(*inv);
+    TORCH_CHECK(inv->scalar_type() == at::kInt && inv->numel() == ids.numel(), "moe_combine: inv");
+    ip = inv->data_ptr<int32_t>();
+  } else {
+    TORCH_CHECK(y.size(0) == T, "moe_combine: y rows");
+  }
+  const c10::DeviceGuard g(out.device());
+  akap_stream::launch_moe_combine(out.data_ptr<float>(), y.data_ptr(), ip, ids.data_ptr<int32_t>(),
+                                  w.data_ptr<float>(), h.data_ptr(), (int)h.stride(0), (int)T,
+                                  (int)out.size(1), (int)ids.size(1), (int)experts, (int)y.size(0),
+                                  is_f32(y, "y"), cur_stream());
+}
+
 }  // namespace
 
 TORCH_LIBRARY(akap_stream, m) {
@@ -266,9 +564,37 @@ TORCH_LIBRARY(akap_stream, m) {
       "sink_attention_decode(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
       "Tensor block_tables, Tensor seq_lens, Tensor? gate, Tensor? sink, float scale, int chunk, "
       "int window, Tensor(b!)? ws_ml, Tensor(c!)? ws_o, int num_parts) -> ()");
+  m.def("add_group_norm(Tensor(a!) out1, Tensor(b!)? out2, Tensor(c!) x, Tensor? y, Tensor? y2, "
+        "Tensor? bias, Tensor w1, Tensor? w2, int groups, float eps) -> ()");
+  m.def("token_shift(Tensor(a!) out, Tensor h, Tensor mu, Tensor(b!) state, Tensor seq_slot, "
+        "Tensor positions) -> ()");
+  m.def("latent_prep(Tensor proj, Tensor(a!) cq_out, Tensor(b!)? cache, Tensor positions, "
+        "Tensor slots, Tensor cos_sin, Tensor q_w, Tensor? kv_w, int q_rank, int kv_rank, "
+        "int rot_dim, int q_off, int kv_off, float eps) -> ()");
+  m.def("rotate_heads(Tensor(a!) q, Tensor positions, Tensor cos_sin, int offset) -> ()");
+  m.def("latent_attention(Tensor(a!) out, Tensor q_lat, Tensor q, int rot_off, Tensor cache, "
+        "Tensor block_tables, Tensor seq_lens, Tensor? q_start, Tensor positions, float scale) "
+        "-> ()");
+  m.def("head_gate(Tensor(a!) out, Tensor o, Tensor gate) -> ()");
+  m.def("xielu(Tensor(a!) out, Tensor x, Tensor? bias, Tensor act) -> ()");
+  m.def("moe_route(Tensor(a!) ids, Tensor(b!) w, Tensor h, Tensor router, Tensor? correction, "
+        "int groups, int keep) -> ()");
+  m.def("relu2_routed(Tensor(a!) out, Tensor up, Tensor ids, Tensor w, int experts) -> ()");
+  m.def("moe_combine(Tensor(a!) out, Tensor y, Tensor? inv, Tensor ids, Tensor w, Tensor h, "
+        "int experts) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(akap_stream, CUDA, m) {
+  m.impl("add_group_norm", &add_group_norm);
+  m.impl("token_shift", &token_shift);
+  m.impl("latent_prep", &latent_prep);
+  m.impl("rotate_heads", &rotate_heads);
+  m.impl("latent_attention", &latent_attention);
+  m.impl("head_gate", &head_gate);
+  m.impl("xielu", &xielu);
+  m.impl("moe_route", &moe_route);
+  m.impl("relu2_routed", &relu2_routed);
+  m.impl("moe_combine", &moe_combine);
   m.impl("embed_scaled", &embed_scaled);
   m.impl("add_norm", &add_norm);
   m.impl("relu2", &relu2);
