@@ -154,3 +154,123 @@ def forward(cfg, W, tokens, want_layers=False):
         streams.append(x.clone())
     logits = group_norm(x, W["final.norm"], groups, eps) @ W["head"].T
     return (logits, torch.stack(streams)) if want_layers else logits
+
+
+# ----------------------------------------------------------------------------- test models
+def make_layer(heads=3, dim=8, rot_dim=4, vdim=6, kv_rank=12, q_rank=10, base=100.0, scale=None,
+               gate="head", kv_from=None, ff=20, moe=None):
+    """One entry of config.json's `layers`.  moe: dict(experts, ff, top, identity, count, keep)
+    for a routed feed-forward; ff None and moe None: no feed-forward."""
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank,
+         "q_rank": q_rank, "rot": {"base": base, "dims": rot_dim},
+         "scale": scale if scale is not None else (dim + rot_dim) ** -0.5}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    if moe is not None:
+        mlp = {"kind": "moe", "expert": {"ff": moe["ff"]},
+               "router": {"experts": moe["experts"], "top": moe["top"],
+                          "identity": moe.get("identity", 0),
+                          "groups": {"count": moe.get("count", 1), "keep": moe.get("keep", 1)}}}
+    elif ff is not None:
+        mlp = {"kind": "dense", "ff": ff}
+    else:
+        mlp = None
+    return {"type": "latent_attention_2" if gate == "element" else "latent_attention", "mixer": m,
+            "mlp": mlp}
+
+
+def make_config(width=24, vocab=41, layers=None, eps=1e-5, groups=3):
+    return {"architecture": "Puputar", "layers": layers, "norm": {"eps": eps, "groups": groups},
+            "vocab": vocab, "width": width}
+
+
+def random_weights(cfg, seed=0):
+    """Random tensors under the checkpoint's names, values that bfloat16 holds exactly."""
+    g = torch.Generator().manual_seed(seed)
+    d = cfg["width"]
+
+    def rnd(*shape, s=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g) * s + mean).to(torch.bfloat16)
+
+    W = {"embed": rnd(cfg["vocab"], d), "embed.norm": rnd(d, s=0.2, mean=1.0),
+         "final.norm": rnd(d, s=0.2, mean=1.0), "head": rnd(cfg["vocab"], d, s=d ** -0.5)}
+    for i, ly in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", ly["mixer"]
+        H, D, r, V, R, Q = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+        W[p + "norm1"] = rnd(d, s=0.2, mean=1.0)
+        W[p + "shift"] = rnd(d, s=0.3, mean=0.4)
+        W[p + "mix.dq"] = rnd(Q, d, s=d ** -0.5)
+        W[p + "mix.dq.norm"] = rnd(Q, s=0.2, mean=1.0)
+        W[p + "mix.uq"] = rnd(H * (D + r), Q, s=2 * Q ** -0.5)
+        if m.get("kv_from") is None:
+            W[p + "mix.dkv"] = rnd(R + r, d, s=d ** -0.5)
+            W[p + "mix.dkv.norm"] = rnd(R, s=0.2, mean=1.0)
+        W[p + "mix.uk"] = rnd(H * D, R, s=2 * R ** -0.5)
+        W[p + "mix.uv"] = rnd(H * V, R, s=R ** -0.5)
+        W[p + "mix.g"] = rnd(H * V if ly["type"] == "latent_attention_2" else H, d, s=d ** -0.5)
+        W[p + "mix.o"] = rnd(d, H * V, s=(H * V) ** -0.5)
+        ml = ly["mlp"]
+        if ml is None:
+            continue
+        W[p + "norm2"] = rnd(d, s=0.2, mean=1.0)
+        if ml["kind"] == "dense":
+            F_ = ml["ff"]
+            W[p + "mlp.up"] = rnd(F_, d, s=d ** -0.5)
+            W[p + "mlp.up.b"] = rnd(F_, s=0.3)
+            W[p + "mlp.down"] = rnd(d, F_, s=F_ ** -0.5)
+            W[p + "mlp.down.b"] = rnd(d, s=0.3)
+            W[p + "mlp.act"] = rnd(2, s=0.7)
+        else:
+            rt, F_ = ml["router"], ml["expert"]["ff"]
+            n = rt["experts"] + rt.get("identity", 0)
+            for e in range(rt["experts"]):
+                W[p + f"mlp.e{e}.up"] = rnd(F_, d, s=d ** -0.5)
+                W[p + f"mlp.e{e}.down"] = rnd(d, F_, s=F_ ** -0.5)
+            W[p + "mlp.router"] = rnd(n, d, s=2 * d ** -0.5)
+            W[p + "mlp.correction"] = rnd(n, s=0.1)
+    return W
+
+
+def decode_step_by_step(cfg, W, tokens):
+    """The same logits computed one token at a time from explicit caches and shift states (an
+    independent check of what a sequence has to carry from step to step)."""
+    W = {k: v.to(F64) for k, v in W.items()}
+    eps, groups = cfg["norm"]["eps"], cfg["norm"]["groups"]
+    L = len(cfg["layers"])
+    prev = [None] * L
+    cache = {}
+    out = []
+    for t, tok in enumerate(tokens):
+        pos = torch.tensor([t])
+        x = group_norm(W["embed"][torch.as_tensor([tok])], W["embed.norm"], groups, eps)
+        for i, ly in enumerate(cfg["layers"]):
+            p, m = f"l{i}.", ly["mixer"]
+            h, prev[i] = token_shift(group_norm(x, W[p + "norm1"], groups, eps), W[p + "shift"],
+                                     prev[i])
+            j = m.get("kv_from")
+            if j is None:
+                c, kr = latent_kv(h, W, p, m, eps, pos)
+                old = cache.get(i)
+                cache[i] = (c, kr) if old is None else (torch.cat([old[0], c]),
+                                                        torch.cat([old[1], kr]))
+                j = i
+            c, kr = cache[j]
+            H, D, r, V = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+            cq = rms(h @ W[p + "mix.dq"].T, eps) * W[p + "mix.dq.norm"]
+            q = (cq @ W[p + "mix.uq"].T).reshape(1, H, D + r)
+            qr = rotate_pairs(q[..., D:], pos, m["rot"]["dims"], m["rot"]["base"])
+            k = (c @ W[p + "mix.uk"].T).reshape(-1, H, D)
+            v = (c @ W[p + "mix.uv"].T).reshape(-1, H, V)
+            s = (torch.einsum("hd,jhd->hj", q[0, :, :D], k) +
+                 torch.einsum("hd,jd->hj", qr[0], kr)) * m["scale"]
+            o = torch.einsum("hj,jhv->hv", torch.softmax(s, dim=-1), v)
+            g = torch.sigmoid(h @ W[p + "mix.g"].T)[0]
+            o = o * (g.reshape(H, V) if ly["type"] == "latent_attention_2" else g[:, None])
+            y = o.reshape(1, H * V) @ W[p + "mix.o"].T
+            ml = ly.get("mlp")
+            if ml is not None:
+                h2 = group_norm(x, W[p + "norm2"], groups, eps)
+                y = y + (dense_ff(h2, W, p) if ml["kind"] == "dense" else moe_ff(h2, W, p, ml))
+            x = x + y
+        out.append(group_norm(x, W["final.norm"], groups, eps) @ W["head"].T)
+    return torch.cat(out)

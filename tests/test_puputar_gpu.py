@@ -1,0 +1,295 @@
+"""Puputar on the HIP kernels: every new kernel against the PyTorch version of the same op (fp32
+and bf16 storage, odd and 16-byte-aligned sizes), then the engine -- mixed steps, hipGraph
+decode, a small page and slot pool -- against the float64 oracle (tests/puputar_oracle.py), and
+greedy generation through LLMEngine.generate."""
+import pytest
+import torch
+
+import puputar_oracle as oracle
+from bidetar_harness import engine, rel_err, replay, tokens, write_model
+from test_puputar import OTHER, _latent_case, base_config
+from aws_k8s_ansible_provisioner_amd.ops import stream as sops
+
+pytestmark = pytest.mark.gpu
+TOL = {"float32": 3e-4, "bfloat16": 0.08}
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def close(a, b, dtype):
+    tol = 2e-5 if dtype == "float32" else 2e-2
+    torch.testing.assert_close(a.float().cpu(), b.float().cpu(), rtol=tol, atol=tol)
+
+
+# ------------------------------------------------------------------ kernels against their ops
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("d,groups", [(24, 4), (2048, 1), (1536, 3), (54, 9), (4100, 2)])
+def test_add_group_norm_kernel(dtype, d, groups):
+    g, dt = gen(d), DT[dtype]
+    T = 7
+    x = torch.randn(T, d, generator=g)
+    y, b = torch.randn(T, d + 3, generator=g).to(dt), torch.randn(d, generator=g).to(dt)
+    y2 = torch.randn(T, d, generator=g)
+    w1, w2 = 1 + 0.3 * torch.randn(d, generator=g), 1 + 0.3 * torch.randn(d, generator=g)
+    for use in [(True, True, True, True), (True, False, False, False), (False, False, False, False),
+                (False, True, True, False)]:
+        xs = [x.clone(), x.clone().cuda()]
+        outs = []
+        for xx in xs:
+            dev = xx.device
+            o1 = torch.zeros(T, d, dtype=dt, device=dev)
+            o2 = torch.zeros(T, d, dtype=dt, device=dev) if use[3] else None
+            sops.stream_add_group_norm(xx, y[:, :d].to(dev) if use[0] else None,
+                                       y2.to(dev) if use[1] else None, b.to(dev) if use[2] else None,
+                                       w1.to(dev), w2.to(dev) if use[3] else None, groups, 1e-5, o1, o2)
+            outs.append((o1, o2))
+        close(xs[1], xs[0], "float32")
+        close(outs[1][0], outs[0][0], dtype)
+        if use[3]:
+            close(outs[1][1], outs[0][1], dtype)
+    # fp32 output from bf16-typed inputs (the normed embedding is the stream itself)
+    o_c, o_g = torch.zeros(T, d), torch.zeros(T, d, device="cuda")
+    sops.stream_add_group_norm(x.clone(), None, None, None, w1, None, groups, 1e-5, o_c)
+    sops.stream_add_group_norm(x.clone().cuda(), None, None, None, w1.cuda(), None, groups, 1e-5, o_g)
+    close(o_g, o_c, "float32")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_token_shift_kernel(dtype):
+    g, dt = gen(1), DT[dtype]
+    d = 70
+    h = torch.randn(9, d, generator=g).to(dt)
+    mu = torch.rand(d, generator=g)
+    state = torch.randn(4, d, generator=g).to(dt)
+    slot = torch.tensor([2, 2, 2, 0, 0, 3, 1, -1, -1], dtype=torch.int32)
+    pos = torch.tensor([5, 6, 7, 0, 1, 9, 4, 0, 0])
+    res = []
+    for dev in ("cpu", "cuda"):
+        st, out = state.clone().to(dev), torch.zeros(9, d, dtype=dt, device=dev)
+        sops.token_shift(h.to(dev), mu.to(dev), st, slot.to(dev), pos.to(dev), out)
+        res.append((out[:7], st))
+    close(res[1][0], res[0][0], dtype)
+    assert torch.equal(res[1][1].cpu(), res[0][1])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("Q,R,r", [(6, 10, 4), (768, 512, 64), (17, 70, 10)])
+def test_latent_prep_and_rotate_kernels(dtype, Q, R, r):
+    g, dt = gen(Q), DT[dtype]
+    T, BS, NB, H, D = 7, 8, 4, 3, 6
+    proj = torch.randn(T, 3 + Q + R + r + 2, generator=g).to(dt)
+    qw, kw = 1 + 0.3 * torch.randn(Q, generator=g), 1 + 0.3 * torch.randn(R, generator=g)
+    pos = torch.tensor([0, 1, 7, 8, 9, 31, 5])
+    slots = torch.tensor([3, 0, 7, 8, 15, 31, -1])
+    table = sops.rotary_table(32, r, 50.0)
+    q = torch.randn(T, H, D + r, generator=g).to(dt)
+    res = []
+    for dev in ("cpu", "cuda"):
+        cq = torch.zeros(T, Q, dtype=dt, device=dev)
+        cache = torch.zeros(NB, BS, R + r, dtype=dt, device=dev)
+        sops.latent_prep(proj.to(dev), cq, cache, pos.to(dev), slots.to(dev), table.to(dev),
+                         qw.to(dev), kw.to(dev), Q, R, r, 3, 3 + Q, 1e-5)
+        cq2 = torch.zeros(T, Q, dtype=dt, device=dev)
+        sops.latent_prep(proj.to(dev), cq2, None, pos.to(dev), slots.to(dev), table.to(dev),
+                         qw.to(dev), None, Q, R, r, 3, -1, 1e-5)
+        assert torch.equal(cq, cq2)
+        qq = q.clone().to(dev)
+        sops.rotate_heads_(qq, pos.to(dev), table.to(dev), D)
+        res.append((cq, cache, qq))
+    for a, b in zip(res[1], res[0]):
+        close(a, b, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,D,r,V,R", [(3, 6, 4, 5, 10), (5, 8, 8, 8, 24), (16, 128, 64, 128, 512),
+                                       (9, 5, 10, 4, 70)])
+def test_latent_attention_kernel(dtype, H, D, r, V, R):
+    dt, BS = DT[dtype], 32
+    lens = [300, 77, 300]
+    cache, bt, rows, w_uk, w_uv, q = _latent_case(H, 23, H, D, r, V, R, BS, lens)
+    pos = torch.cat([torch.arange(280, 300), torch.tensor([76, 299, 0])])
+    q_start = torch.tensor([0, 20, 21, 22, 23], dtype=torch.int32)
+    seq_lens = torch.tensor([300, 77, 300, 0], dtype=torch.int32)
+    bt = torch.cat([bt, bt[:1]])
+    cache[int(bt[0, 0]), 5] *= 4.0          # a far key that matters
+    q_lat = (torch.einsum("thd,hdr->htr", q[..., :D], w_uk) * R ** -0.5).contiguous()
+    scale = (D + r) ** -0.5
+    res = []
+    for dev in ("cpu", "cuda"):
+        out = torch.zeros(H, 23, R, dtype=dt, device=dev)
+        sops.latent_attention(out, q_lat.to(dt).to(dev), q.to(dt).to(dev), D, cache.to(dt).to(dev),
+                              bt.to(dev), seq_lens.to(dev), q_start.to(dev), pos.to(dev), scale)
+        out1 = torch.zeros(H, 3, R, dtype=dt, device=dev)
+        sops.latent_attention(out1, q_lat[:, 20:23].contiguous().to(dt).to(dev),
+                              q[20:23].contiguous().to(dt).to(dev), D, cache.to(dt).to(dev),
+                              bt[1:4].contiguous().to(dev), seq_lens[1:4].contiguous().to(dev), None,
+                              pos[20:23].to(dev), scale)
+        res.append((out, out1))
+    close(res[1][0], res[0][0], dtype)
+    close(res[1][1], res[0][1], dtype)
+    close(res[1][1][:, :2], res[1][0][:, 20:22], dtype)
+    assert res[1][0][:, 22].abs().max().item() == 0      # padding rows are left alone
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gate_activation_and_routing_kernels(dtype):
+    g, dt = gen(4), DT[dtype]
+    H, T, V, F_ = 3, 6, 5, 37
+    o = torch.randn(H, T, V, generator=g).to(dt)
+    wide = torch.randn(T, 2 + H * V + 1, generator=g).to(dt)
+    x = (torch.randn(T, F_ + 2, generator=g) * 3).to(dt)
+    b = torch.randn(F_, generator=g).to(dt)
+    act = torch.tensor([-0.7, 1.3])
+    n, d, E = 12, 40, 9
+    h = torch.randn(T, d, generator=g).to(dt)
+    router, corr = torch.randn(n, d, generator=g), torch.randn(n, generator=g) * 0.1
+    up = torch.randn(T, E * F_, generator=g).to(dt)
+    ys = torch.randn(T * 4, d, generator=g).to(dt)
+    res = []
+    for dev in ("cpu", "cuda"):
+        r = []
+        for cols in (H, H * V):
+            out = torch.zeros(T, H * V + 3, dtype=dt, device=dev)
+            sops.head_gate(o.to(dev), wide[:, 2:2 + cols].to(dev), out[:, :H * V])
+            r.append(out)
+        out = torch.zeros(T, F_ + 1, dtype=dt, device=dev)
+        sops.xielu(x[:, 1:1 + F_].to(dev), b.to(dev), act.to(dev), out[:, :F_])
+        r.append(out)
+        for count, keep, top in [(1, 1, 4), (3, 2, 4), (4, 1, 3), (12, 5, 4)]:
+            ids, w = sops.moe_route(h.to(dev), router.to(dev), corr.to(dev), top, count, keep)
+            order = ids.long().argsort(dim=1)
+            r += [ids.long().gather(1, order).float(), w.gather(1, order)]
+        ids, w = sops.moe_route(h.to(dev), router.to(dev), corr.to(dev), 4, 3, 2)
+        a = torch.zeros(T, E * F_, dtype=dt, device=dev)
+        sops.relu2_routed(up.to(dev), ids, w, E, a)
+        r.append(a)
+        inv = torch.randperm(T * 4, generator=gen(5)).int().view(T, 4).to(dev)
+        for iv, y in ((None, ys[:T]), (inv, ys)):
+            c = torch.zeros(T, d, device=dev)
+            sops.moe_combine(c, y.contiguous().to(dev), iv, ids, w, h.to(dev), E)
+            r.append(c)
+        res.append(r)
+    for a, b_ in zip(res[1], res[0]):
+        close(a, b_, dtype if a.dtype != torch.float32 or dtype == "float32" else "bfloat16")
+
+
+# ------------------------------------------------------------------ the engine on the GPU
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    cfg = base_config()
+    W = oracle.random_weights(cfg, seed=2)
+    reqs = {"a": tokens(75, cfg["vocab"], 1), "b": tokens(41, cfg["vocab"], 2),
+            "c": tokens(23, cfg["vocab"], 3), "d": tokens(1, cfg["vocab"], 4),
+            "e": tokens(64, cfg["vocab"], 5)}
+    want = {n: oracle.forward(cfg, W, t) for n, t in reqs.items()}
+    return cfg, W, write_model(tmp_path_factory.mktemp("puputar_gpu"), cfg, W), reqs, want
+
+
+def check(got, want, dtype):
+    for n in got:
+        e = rel_err(got[n], want[n])
+        if dtype == "bfloat16":
+            # a close routing choice can flip at bf16 precision and move one position's logits
+            # (and, through the cache, a little of what follows): nearly all must be close
+            assert e.median().item() < 0.03 and (e > TOL[dtype]).sum().item() <= 2, \
+                f"{n}: {(e > TOL[dtype]).sum().item()} positions off, worst {e.max():.2e}"
+        else:
+            assert e.max().item() < TOL[dtype], f"{n}: position {int(e.argmax())} off by {e.max():.2e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("eager", [False, True])
+def test_schedules(model, dtype, eager):
+    _, _, path, reqs, want = model
+    eng = engine(path, dtype=dtype, device="cuda", eager=eager)
+    assert eager or eng.runner.graphs, "decode hipGraphs were not captured"
+    one = {"a": reqs["a"]}
+    check(replay(eng, reqs, [[(n, len(t))] for n, t in reqs.items()]), want, dtype)
+    check(replay(eng, one, [[("a", 40)]] + [[("a", 1)]] * 35), want, dtype)
+    check(replay(eng, one, [[("a", s)] for s in [3, 2, 7, 2, 19, 2, 5, 33, 2]]), want, dtype)
+    sched = [[("a", 30), ("b", 2), ("c", 1)],
+             [("a", 1), ("b", 20), ("c", 22), ("d", 1)],
+             [("a", 1), ("b", 1), ("e", 33)],
+             [("a", 1), ("b", 1)],
+             [("b", 17), ("e", 1)],
+             [("a", 42), ("e", 30)]]
+    check(replay(eng, reqs, sched), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_small_pool_is_used_again(model, dtype):
+    _, _, path, reqs, want = model
+    eng = engine(path, dtype=dtype, max_tokens=160, max_seqs=2, device="cuda")
+    many = {f"{n}{i}": reqs[n] for i in range(2) for n in ("b", "c", "e")}
+    many["a"] = reqs["a"]
+    sched = [[("b0", 41), ("c0", 23)], [("e0", 64), ("c1", 22)], [("c1", 1)],
+             [("a", 75), ("b1", 41)], [("e1", 10)], [("e1", 54)]]
+    for _ in range(2):  # graphs replayed again over pages and slots that changed owners
+        check(replay(eng, many, sched), {k: want[k[0]] for k in many}, dtype)
+    assert eng.sched.num_free_blocks() == 5 and eng.sched.num_free_tail_slots == 2
+
+
+def test_long_decode_through_graphs(tmp_path):
+    cfg = oracle.make_config(width=64, vocab=37, groups=2, layers=[
+        oracle.make_layer(heads=4, dim=16, rot_dim=8, vdim=16, kv_rank=24, q_rank=20),
+        oracle.make_layer(heads=2, dim=8, rot_dim=8, vdim=12, kv_rank=24, q_rank=16, kv_from=0,
+                          gate="element",
+                          moe=dict(experts=6, ff=16, top=2, identity=2, count=4, keep=2))])
+    W = oracle.random_weights(cfg, seed=5)
+    toks = tokens(700, 37, 6)
+    want = {"a": oracle.forward(cfg, W, toks)}
+    eng = engine(write_model(tmp_path, cfg, W), dtype="float32", max_tokens=704, device="cuda")
+    assert eng.runner.graphs
+    check(replay(eng, {"a": toks}, [[("a", 500)]] + [[("a", 1)]] * 200), want, "float32")
+
+
+def test_large_prompt_takes_the_sorted_expert_path(tmp_path):
+    """A prompt portion over the small-batch threshold of the routed feed-forward."""
+    from aws_k8s_ansible_provisioner_amd.models import puputar
+
+    cfg = oracle.make_config(width=32, vocab=37, groups=1, layers=[
+        oracle.make_layer(heads=2, dim=8, rot_dim=4, vdim=8, kv_rank=16, q_rank=12,
+                          moe=dict(experts=5, ff=16, top=2, identity=1, count=3, keep=2))])
+    W = oracle.random_weights(cfg, seed=6)
+    toks = tokens(puputar.MOE_DENSE_ROWS + 70, 37, 7)
+    want = {"a": oracle.forward(cfg, W, toks)}
+    eng = engine(write_model(tmp_path, cfg, W), dtype="float32", max_tokens=512, device="cuda")
+    n = puputar.MOE_DENSE_ROWS + 40
+    check(replay(eng, {"a": toks}, [[("a", n)], [("a", 30)]]), want, "float32")
+
+
+def test_greedy_generation(model):
+    from aws_k8s_ansible_provisioner_amd.engine.config import EngineConfig, SamplingParams
+    from aws_k8s_ansible_provisioner_amd.engine.llm_engine import LLMEngine
+
+    cfg, W, path, _, _ = model
+    eng = LLMEngine(EngineConfig(model=path, load_format="safetensors", weights_path=path,
+                                 dtype="float32", max_model_len=128, max_num_seqs=4,
+                                 max_num_batched_tokens=24, num_gpu_blocks=16, device="cuda",
+                                 gc_freeze=False), log=lambda *a: None)
+    assert eng.runner.graphs
+    prompts = [tokens(n, cfg["vocab"], 20 + n) for n in (30, 3, 17, 9)]
+    outs = eng.generate(None, SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True),
+                        prompt_ids=prompts)
+    assert [len(o.output_ids) for o in outs] == [12] * 4
+    for p, o in zip(prompts, outs):
+        logits = oracle.forward(cfg, W, p + o.output_ids)
+        for i, tok in enumerate(o.output_ids):
+            row = logits[len(p) - 1 + i]
+            assert row[tok] >= row.max() - 1e-3 * row.std(), (i, tok, int(row.argmax()))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(OTHER))
+def test_other_configurations(tmp_path, name, dtype):
+    cfg = oracle.make_config(**dict(OTHER[name]))
+    W = oracle.random_weights(cfg, seed=len(name))
+    reqs = {"p": tokens(45, cfg["vocab"], 11), "q": tokens(38, cfg["vocab"], 12)}
+    want = {n: oracle.forward(cfg, W, t) for n, t in reqs.items()}
+    eng = engine(write_model(tmp_path, cfg, W), dtype=dtype, device="cuda")
+    sched = [[("p", 17), ("q", 2)], [("p", 1), ("q", 30)], [("p", 27), ("q", 1)],
+             [("q", 1)], [("q", 4)]]
+    check(replay(eng, reqs, sched), want, dtype)
