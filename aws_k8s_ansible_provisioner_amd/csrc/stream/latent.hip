@@ -142,7 +142,13 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(LatentPrepParams p) {
   ss = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)p.kv_rank + p.eps);
   T* dst = (T*)p.cache + (size_t)slot * (p.kv_rank + p.rot_dim);
-  for (int c = threadIdx.x; c < p.kv_rank; c += 256) stf(dst + c, ldf(kv + c) * inv * p.kv_w[c]);
+  // the grouped copy: 8 consecutive tokens of one dimension are 16 contiguous bytes
+  T* grp = p.vgroups ? (T*)p.vgroups + (size_t)(slot >> 3) * p.kv_rank * 8 + (slot & 7) : nullptr;
+  for (int c = threadIdx.x; c < p.kv_rank; c += 256) {
+    const T v = (T)(ldf(kv + c) * inv * p.kv_w[c]);
+    dst[c] = v;
+    if (grp) grp[(size_t)c * 8] = v;
+  }
   int64_t pos = p.positions[t];
   pos = pos < 0 ? 0 : (pos >= p.max_pos ? p.max_pos - 1 : pos);
   const float* cs = p.cos_sin + (size_t)pos * p.rot_dim;

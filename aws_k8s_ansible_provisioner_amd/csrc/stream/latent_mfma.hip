@@ -1,0 +1,347 @@
+// Matrix-core latent attention (bf16): every head against ONE cached row per key.
+//
+// A cached token is a row [c (R) | k_rot (r)] of the latent cache, and its latent c a second time
+// in 8-token groups [NB BS / 8, R, 8] (dimension-major inside a group).  With the unrotated query
+// already multiplied into the latent space, head h's score of key j is
+// q_lat[h] . c_j + q_rot[h] . k_rot_j and its output sum_j p_j c_j: a multi-query attention with
+// R + r score dimensions and R value dimensions, whatever the number of heads.
+//
+// v_mfma_f32_32x32x16_bf16 computes S^T = K Q^T (keys are the 32 rows, queries the 32 columns)
+// and O^T = C^T P^T.  A query is a lane column, so its softmax statistics are 16 registers and
+// one exchange between the lane halves.  The K rows are loaded in the order (bits 2 and 3 of
+// the row swapped) that makes a lane's S^T accumulators exactly the 8 keys of one group, so P
+// moves from accumulator to operand without lane traffic and the C^T operand is one 16-byte
+// load from the grouped copy.  The query tile (32 columns x (R + r)) lives in LDS: at R = 512
+// the output accumulators alone are 256 registers.  K and C fragments come straight from
+// global memory (L1 / L2: the heads of a token tile are workgroups of one XCD).
+//
+// Prefill: a wave owns 32 consecutive tokens of one head (causal mask only in the blocks that
+// cross its positions).  Decode: the 32 columns are the heads of one token; the key range is
+// cut into partitions merged by a second launch.
+#include "../kernels/common.h"
+#include "stream.h"
+
+namespace akap_stream {
+
+using akap::bf16;
+using akap::bf16x8;
+using akap::f32x16;
+
+namespace {
+
+__device__ __forceinline__ int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
+
+template <int NV>
+struct LatentState {
+  f32x16 o[NV];
+  float m, l;   // m in log2 units of the scaled scores
+};
+
+// LDS row pitch of the query tile (elements): 16 bytes of padding per row
+__host__ __device__ constexpr int q_pitch(int DK) { return DK + 8; }
+
+// The wave's 32 query columns -> LDS [32][pitch]: column col is token tok[col] of head h,
+// [q_lat[h, tok] (R) | q[tok, h, rot_off : rot_off + r]].
+template <int NV, int NKR>
+__device__ __forceinline__ void load_queries(bf16* qs, const LatentAttnParams& p, int h, int my_tok) {
+  constexpr int R = 32 * NV, DK = R + 16 * NKR, CH = DK / 8, P = q_pitch(DK);
+  const int lane = threadIdx.x & 63;
+  for (int idx = lane; idx < 32 * CH; idx += 64) {
+    const int col = idx / CH, ch = idx - col * CH;
+    const int t = __shfl(my_tok, col, 64);
+    const bf16* src = ch * 8 < R
+        ? (const bf16*)p.q_lat + ((size_t)h * p.T + t) * R + ch * 8
+        : (const bf16*)p.q + (size_t)t * p.q_stride + (size_t)h * p.q_head + p.rot_off + ch * 8 - R;
+    *reinterpret_cast<bf16x8*>(qs + col * P + ch * 8) = *reinterpret_cast<const bf16x8*>(src);
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+// Keys [jb, je] (jb a multiple of 32) against the wave's 32 columns; pos: this lane's column's
+// position (keys above it are masked); pos_min: the smallest position among the columns.
+template <int NV, int NKR>
+__device__ __forceinline__ void attend(LatentState<NV>& st, const LatentAttnParams& p,
+                                       const int32_t* __restrict__ bt, const bf16* qs, int pos,
+                                       int pos_min, int jb, int je) {
+  constexpr int R = 32 * NV, DK = R + 16 * NKR, KS = DK / 16, P = q_pitch(DK);
+  const float sc2 = p.scale * 1.44269504088896f;
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 31, hf = lane >> 5;
+  const int krow = swap23(col);
+  const bf16* cache = (const bf16*)p.cache;
+  const bf16* vg = (const bf16*)p.vgroups;
+  const bf16* qcol = qs + col * P + 8 * hf;
+  for (int j0 = jb; j0 <= je; j0 += 32) {
+    const int bi = j0 / p.BS;
+    int blk = bi < p.max_blocks ? bt[bi] : 0;
+    if (blk < 0 || blk >= p.NB) blk = 0;
+    const size_t row0 = (size_t)blk * p.BS + (j0 - bi * p.BS);   // a multiple of 32
+    const bf16* kp = cache + (row0 + krow) * DK + 8 * hf;
+    f32x16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+    for (int c = 0; c < KS; ++c) {
+      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + 16 * c);
+      const bf16x8 qf = *reinterpret_cast<const bf16x8*>(qcol + 16 * c);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf, s, 0, 0, 0);
+    }
+    // accumulator register i of this lane: key j0 + 16 (i >> 3) + 8 hf + (i & 7), column col
+    float sv[16];
+    float bmax = -INFINITY;
+    if (j0 + 31 <= pos_min) {       // (wave-uniform) visible to every column
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        sv[i] = s[i];
+        bmax = fmaxf(bmax, sv[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = j0 + 16 * (i >> 3) + 8 * hf + (i & 7);
+        sv[i] = key <= pos ? s[i] : -INFINITY;
+        bmax = fmaxf(bmax, sv[i]);
+      }
+    }
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    const float mn = fmaxf(st.m, bmax * sc2);
+    const float ms = mn == -INFINITY ? 0.f : mn;   // nothing visible yet: every exp below is 0
+    const float alpha = __builtin_amdgcn_exp2f(st.m - ms);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -ms));
+      psum += sv[i];
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    st.l = st.l * alpha + psum;
+    st.m = mn;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) pb[i >> 3][i & 7] = (bf16)sv[i];
+    if (__any(alpha != 1.0f)) {     // (wave-uniform) the maxima settle after the first blocks
+#pragma unroll
+      for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) st.o[dt][i] *= alpha;
+    }
+    // latent groups of this block: row0 / 8 is its first group
+    const bf16* vp = vg + (((row0 >> 3) + hf) * R + col) * 8;
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt) {
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl) {
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vp + ((size_t)(2 * sl) * R + 32 * dt) * 8);
+        st.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[sl], st.o[dt], 0, 0, 0);
+      }
+    }
+  }
+}
+
+template <int NV>
+__device__ __forceinline__ void init(LatentState<NV>& st) {
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) st.o[dt][i] = 0.f;
+}
+
+// accumulator register i of o[dt]: dimension 32 dt + 8 (i >> 2) + 4 hf + (i & 3)
+template <int NV>
+__device__ __forceinline__ void store(const LatentState<NV>& st, bf16* o) {
+  const int hf = (threadIdx.x & 63) >> 5;
+  const float f = st.l > 0.f ? 1.0f / st.l : 0.f;
+#pragma unroll
+  for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; i += 4) {
+      akap::bf16x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (bf16)(st.o[dt][i + e] * f);
+      *reinterpret_cast<akap::bf16x4*>(o + 32 * dt + 8 * (i >> 2) + 4 * hf) = v;
+    }
+}
+
+// Prefill: flat grid over (32-token sub-tile, head block) units, WPB waves (heads) per workgroup
+template <int NV, int NKR, int WPB>
+__global__ __launch_bounds__(64 * WPB) void latent_prefill_mfma_kernel(LatentAttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int R = 32 * NV, DK = R + 16 * NKR, P = q_pitch(DK);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int col = lane & 31;
+  // the hardware deals workgroup i to XCD i % 8: units (sub-tiles, longest first) are dealt
+  // round-robin over the XCDs, and the head blocks of one unit are workgroups of ONE XCD, so
+  // a token tile's cached rows cross into a single L2
+  const int hblocks = (p.H + WPB - 1) / WPB;
+  const int sub = p.tile_rows / 32;
+  const int xcd = blockIdx.x & 7, jx = blockIdx.x >> 3;
+  const int unit = (jx / hblocks) * 8 + xcd;
+  if (unit >= p.num_tiles * sub) return;
+  const int h = (jx % hblocks) * WPB + wave;
+  if (h >= p.H) return;                          // no workgroup barriers below
+  // the scheduler sorts tiles by ascending causal work: walk from the end
+  const int tile = p.num_tiles - 1 - unit / sub;
+  const int si = sub - 1 - unit % sub;
+  const int b = p.tile_seq[tile];
+  if (b < 0 || b >= p.B) return;
+  const int qs0 = p.q_start[b];
+  const int qlen = p.q_start[b + 1] - qs0;
+  const int kv = p.seq_lens[b];
+  const int rend = min(p.tile_row[tile] + p.tile_rows, qlen);
+  const int r0 = p.tile_row[tile] + 32 * si;
+  if (r0 >= rend || kv < qlen) return;
+  const int r = r0 + col;
+  const bool valid = r < rend;
+  const int t = qs0 + (valid ? r : r0);
+  const int pos = kv - qlen + r;
+  bf16* qs = reinterpret_cast<bf16*>(smem) + (size_t)wave * 32 * P;
+  load_queries<NV, NKR>(qs, p, h, t);
+  LatentState<NV> st;
+  init(st);
+  const int pos_first = kv - qlen + r0;
+  const int pos_last = kv - qlen + min(r0 + 31, rend - 1);
+  attend<NV, NKR>(st, p, p.block_tables + (size_t)b * p.max_blocks, qs, pos, pos_first, 0,
+                  pos_last);
+  if (valid) store<NV>(st, (bf16*)p.out + ((size_t)h * p.T + t) * R);
+}
+
+// Decode: grid (B, ceil(H / 32), parts), one wave; columns are heads
+template <int NV, int NKR>
+__global__ __launch_bounds__(64) void latent_decode_mfma_kernel(LatentAttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int R = 32 * NV;
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 31, hf = lane >> 5;
+  const int b = blockIdx.x, part = blockIdx.z;
+  const int c0 = blockIdx.y * 32;
+  const int kv = p.seq_lens[b];
+  if (kv <= 0) return;                           // a padding row: nothing read or written
+  const bool valid = c0 + col < p.H;
+  const int h = valid ? c0 + col : c0;
+  const int pos1 = kv - 1;
+  int per = (pos1 + 1 + p.num_parts - 1) / p.num_parts;
+  per = (per + 31) & ~31;
+  const int jb = part * per;
+  const int je = min(pos1, jb + per - 1);
+  bf16* qs = reinterpret_cast<bf16*>(smem);
+  LatentState<NV> st;
+  init(st);
+  if (jb <= je) {
+    // column col is head c0 + col of token b: per-column head, one token
+    {
+      constexpr int DK = R + 16 * NKR, CH = DK / 8, P = q_pitch(DK);
+      for (int idx = lane; idx < 32 * CH; idx += 64) {
+        const int cc = idx / CH, ch = idx - cc * CH;
+        const int hh = c0 + cc < p.H ? c0 + cc : c0;
+        const bf16* src = ch * 8 < R
+            ? (const bf16*)p.q_lat + ((size_t)hh * p.T + b) * R + ch * 8
+            : (const bf16*)p.q + (size_t)b * p.q_stride + (size_t)hh * p.q_head + p.rot_off +
+                  ch * 8 - R;
+        *reinterpret_cast<bf16x8*>(qs + cc * P + ch * 8) = *reinterpret_cast<const bf16x8*>(src);
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+    attend<NV, NKR>(st, p, p.block_tables + (size_t)b * p.max_blocks, qs, pos1, pos1, jb, je);
+  }
+  if (!valid) return;
+  if (p.num_parts == 1) {
+    store<NV>(st, (bf16*)p.out + ((size_t)h * p.T + b) * R);
+    return;
+  }
+  const size_t slot = ((size_t)b * p.H + h) * p.num_parts + part;
+  if (hf == 0) {
+    p.ws_ml[slot * 2] = st.m;
+    p.ws_ml[slot * 2 + 1] = st.l;
+  }
+#pragma unroll
+  for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      p.ws_o[slot * R + 32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = st.o[dt][i];
+}
+
+// grid (B, H): merge the partitions of one (token, head)
+__global__ __launch_bounds__(64) void latent_decode_merge_kernel(LatentAttnParams p) {
+  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  if (p.seq_lens[b] <= 0) return;
+  const size_t base = ((size_t)b * p.H + h) * p.num_parts;
+  float m = -INFINITY;
+  for (int i = 0; i < p.num_parts; ++i)
+    if (p.ws_ml[(base + i) * 2 + 1] > 0.f) m = fmaxf(m, p.ws_ml[(base + i) * 2]);
+  float l = 0.f;
+  for (int i = 0; i < p.num_parts; ++i) {
+    const float li = p.ws_ml[(base + i) * 2 + 1];
+    if (li > 0.f) l += li * __builtin_amdgcn_exp2f(p.ws_ml[(base + i) * 2] - m);
+  }
+  const float f = l > 0.f ? 1.0f / l : 0.f;
+  bf16* o = (bf16*)p.out + ((size_t)h * p.T + b) * p.R;
+  for (int d = lane; d < p.R; d += 64) {
+    float a = 0.f;
+    for (int i = 0; i < p.num_parts; ++i) {
+      const float li = p.ws_ml[(base + i) * 2 + 1];
+      if (li > 0.f)
+        a += p.ws_o[(base + i) * p.R + d] * __builtin_amdgcn_exp2f(p.ws_ml[(base + i) * 2] - m);
+    }
+    o[d] = (bf16)(a * f);
+  }
+}
+
+template <int NV, int NKR>
+void launch_prefill(const LatentAttnParams& p, hipStream_t s) {
+  constexpr int DK = 32 * NV + 16 * NKR;
+  constexpr size_t per_wave = (size_t)32 * q_pitch(DK) * sizeof(bf16);
+  const int units = p.num_tiles * (p.tile_rows / 32);
+  // as many heads per workgroup as fit 64 KB of LDS
+  if (4 * per_wave <= 64 * 1024) {
+    const unsigned grid = (unsigned)((units + 7) / 8 * 8) * ((p.H + 3) / 4);
+    latent_prefill_mfma_kernel<NV, NKR, 4><<<grid, 256, 4 * per_wave, s>>>(p);
+  } else if (2 * per_wave <= 64 * 1024) {
+    const unsigned grid = (unsigned)((units + 7) / 8 * 8) * ((p.H + 1) / 2);
+    latent_prefill_mfma_kernel<NV, NKR, 2><<<grid, 128, 2 * per_wave, s>>>(p);
+  } else {
+    const unsigned grid = (unsigned)((units + 7) / 8 * 8) * p.H;
+    latent_prefill_mfma_kernel<NV, NKR, 1><<<grid, 64, per_wave, s>>>(p);
+  }
+}
+
+template <int NV, int NKR>
+void launch_decode(const LatentAttnParams& p, hipStream_t s) {
+  constexpr int DK = 32 * NV + 16 * NKR;
+  const dim3 grid(p.B, (p.H + 31) / 32, p.num_parts);
+  latent_decode_mfma_kernel<NV, NKR><<<grid, 64, (size_t)32 * q_pitch(DK) * sizeof(bf16), s>>>(p);
+  if (p.num_parts > 1) latent_decode_merge_kernel<<<dim3(p.B, p.H), 64, 0, s>>>(p);
+}
+
+}  // namespace
+
+// the latent / rotated sizes the matrix kernels are built for
+bool latent_mfma_sizes(int R, int r) {
+  const int nv = R / 32, nkr = r / 16;
+  if (R % 32 || r % 16) return false;
+  return (nv == 2 && nkr == 1) || (nv == 3 && nkr == 1) || (nv == 4 && (nkr == 1 || nkr == 2)) ||
+         (nv == 8 && (nkr == 2 || nkr == 4)) || (nv == 16 && nkr == 4);
+}
+
+#define LATENT_SIZES(F)                                                                    \
+  const int nv = p.R / 32, nkr = p.r / 16;                                                 \
+  if (nv == 2 && nkr == 1) F<2, 1>(p, s);                                                  \
+  else if (nv == 3 && nkr == 1) F<3, 1>(p, s);                                             \
+  else if (nv == 4 && nkr == 1) F<4, 1>(p, s);                                             \
+  else if (nv == 4 && nkr == 2) F<4, 2>(p, s);                                             \
+  else if (nv == 8 && nkr == 2) F<8, 2>(p, s);                                             \
+  else if (nv == 8 && nkr == 4) F<8, 4>(p, s);                                             \
+  else if (nv == 16 && nkr == 4) F<16, 4>(p, s);
+
+void launch_latent_prefill_mfma(const LatentAttnParams& p, hipStream_t s) {
+  if (p.num_tiles <= 0 || p.H <= 0) return;
+  LATENT_SIZES(launch_prefill)
+}
+
+void launch_latent_decode_mfma(const LatentAttnParams& p, hipStream_t s) {
+  if (p.B <= 0 || p.H <= 0) return;
+  LATENT_SIZES(launch_decode)
+}
+
+}  // namespace akap_stream

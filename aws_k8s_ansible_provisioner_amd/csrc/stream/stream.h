@@ -85,6 +85,7 @@ struct LatentPrepParams {
   int proj_stride;
   void* cq_out;       // [T, q_rank]
   void* cache;        // [NB * BS, kv_rank + rot_dim] or null
+  void* vgroups;      // [NB * BS / 8, kv_rank, 8]: the latent again, in 8-token groups, or null
   const int64_t* positions;
   const int64_t* slots;
   const float* cos_sin;  // [max_pos, rot_dim] = [cos | sin]
@@ -115,8 +116,21 @@ struct LatentAttnParams {
   float scale;
   int T, B, H, R, r, BS;
   int vec;              // rows of the cache can be read in 16-byte pieces
+  // matrix-core kernels only
+  const void* vgroups;          // [NB * BS / 8, R, 8]
+  int NB;
+  const int32_t* tile_seq;      // prefill tile map: sequence and first chunk row of a tile
+  const int32_t* tile_row;
+  int num_tiles, tile_rows;
+  float* ws_ml;                 // decode split: (max, sum) [B, H, parts, 2]
+  float* ws_o;                  //               outputs    [B, H, parts, R]
+  int num_parts;
 };
 void launch_latent_attention(const LatentAttnParams& p, bool f32, hipStream_t s);
+// bf16, R / r among the built sizes (latent_mfma_sizes), BS % 32 == 0, 16-byte aligned rows
+bool latent_mfma_sizes(int R, int r);
+void launch_latent_prefill_mfma(const LatentAttnParams& p, hipStream_t s);
+void launch_latent_decode_mfma(const LatentAttnParams& p, hipStream_t s);
 
 void launch_head_gate(void* out, int out_stride, const void* o, const void* gate, int gate_stride,
                       bool per_head, int rows, int H, int V, bool f32, hipStream_t s);

@@ -332,7 +332,7 @@ void token_shift(Tensor out, Tensor h, Tensor mu, Tensor state, Tensor seq_slot,
 void latent_prep(Tensor proj, Tensor cq_out, std::optional<Tensor> cache, Tensor positions,
                  Tensor slots, Tensor cos_sin, Tensor q_w, std::optional<Tensor> kv_w,
                  int64_t q_rank, int64_t kv_rank, int64_t rot_dim, int64_t q_off, int64_t kv_off,
-                 double eps) {
+                 double eps, std::optional<Tensor> vgroups) {
   CHECK_GPU(proj); CHECK_LAST_CONTIG(proj); CHECK_GPU(cq_out); CHECK_CONTIG(cq_out);
   CHECK_GPU(positions); CHECK_GPU(slots); CHECK_CONTIG(positions); CHECK_CONTIG(slots);
   CHECK_GPU(cos_sin); CHECK_F32(cos_sin); CHECK_CONTIG(cos_sin);
@@ -370,6 +370,13 @@ void latent_prep(Tensor proj, Tensor cq_out, std::optional<Tensor> cache, Tensor
     p.cache = cache->data_ptr();
     p.kv_w = kv_w->data_ptr<float>();
     p.num_slots = cache->size(0) * cache->size(1);
+    if (vgroups.has_value()) {
+      CHECK_GPU(*vgroups); CHECK_CONTIG(*vgroups);
+      TORCH_CHECK(vgroups->scalar_type() == cache->scalar_type() && cache->size(1) % 8 == 0 &&
+                      vgroups->numel() == cache->size(0) * cache->size(1) * kv_rank,
+                  "latent groups must be [NB, BS / 8, R, 8]");
+      p.vgroups = vgroups->data_ptr();
+    }
   }
   const c10::DeviceGuard g(proj.device());
   akap_stream::launch_latent_prep(p, f32, cur_stream());
@@ -442,6 +449,99 @@ void latent_attention(Tensor out, Tensor q_lat, Tensor q, int64_t rot_off, Tenso
   TORCH_CHECK((H + 3) / 4 <= 65535, "too many heads");
   const c10::DeviceGuard g(q.device());
   akap_stream::launch_latent_attention(p, f32, cur_stream());
+}
+
+// operands common to the two matrix-core launches
+akap_stream::LatentAttnParams latent_mfma_params(const Tensor& out, const Tensor& q_lat,
+                                                 const Tensor& q, int64_t rot_off,
+                                                 const Tensor& cache, const Tensor& vgroups,
+                                                 const Tensor& block_tables,
+                                                 const Tensor& seq_lens, double scale) {
+  CHECK_GPU(out); CHECK_GPU(q_lat); CHECK_GPU(q); CHECK_GPU(cache); CHECK_GPU(vgroups);
+  CHECK_GPU(block_tables); CHECK_GPU(seq_lens);
+  CHECK_CONTIG(out); CHECK_CONTIG(q_lat); CHECK_CONTIG(cache); CHECK_CONTIG(vgroups);
+  CHECK_CONTIG(seq_lens);
+  for (const Tensor* t : {&out, &q_lat, &q, &cache, &vgroups})
+    TORCH_CHECK(t->scalar_type() == at::kBFloat16, "matrix-core latent attention is bf16");
+  TORCH_CHECK(q_lat.dim() == 3 && out.sizes() == q_lat.sizes() && q.dim() == 3 &&
+                  q.stride(2) == 1 && q.stride(1) == q.size(2), "latent attention: q shapes");
+  const int64_t H = q_lat.size(0), T = q_lat.size(1), R = q_lat.size(2);
+  TORCH_CHECK(q.size(0) == T && q.size(1) == H, "latent attention: q is [T, H, n]");
+  TORCH_CHECK(cache.dim() == 3 && cache.size(2) > R, "latent cache [NB, BS, R + r]");
+  const int64_t r = cache.size(2) - R, BS = cache.size(1);
+  TORCH_CHECK(akap_stream::latent_mfma_sizes((int)R, (int)r) && BS % 32 == 0,
+              "latent sizes / block size not built for the matrix cores");
+  TORCH_CHECK(vgroups.numel() == cache.size(0) * BS * R, "latent groups [NB, BS / 8, R, 8]");
+  TORCH_CHECK(rot_off >= 0 && rot_off + r <= q.size(2) && rot_off % 8 == 0 && q.size(2) % 8 == 0 &&
+                  q.stride(0) % 8 == 0 && scale > 0, "rotated query part: place / alignment");
+  for (const Tensor* t : {&q_lat, &q, &cache, &vgroups})
+    TORCH_CHECK((uintptr_t)t->data_ptr() % 16 == 0, "operands must be 16-byte aligned");
+  TORCH_CHECK(block_tables.dim() == 2 && block_tables.scalar_type() == at::kInt &&
+                  block_tables.stride(1) == 1 && seq_lens.scalar_type() == at::kInt &&
+                  block_tables.size(0) >= seq_lens.numel(), "block_tables / seq_lens");
+  TORCH_CHECK(cache.size(0) * BS < (1LL << 31), "cache has too many rows");
+  akap_stream::LatentAttnParams p{};
+  p.out = out.data_ptr();
+  p.q_lat = q_lat.data_ptr();
+  p.q = q.data_ptr();
+  p.q_stride = q.stride(0);
+  p.q_head = q.size(2);
+  p.rot_off = rot_off;
+  p.cache = cache.data_ptr();
+  p.vgroups = vgroups.data_ptr();
+  p.NB = cache.size(0);
+  p.block_tables = block_tables.data_ptr<int32_t>();
+  p.max_blocks = block_tables.stride(0);
+  p.seq_lens = seq_lens.data_ptr<int32_t>();
+  p.scale = (float)scale;
+  p.T = T; p.B = seq_lens.numel(); p.H = H; p.R = R; p.r = r; p.BS = BS;
+  p.num_parts = 1;
+  return p;
+}
+
+void latent_attention_prefill_mfma(Tensor out, Tensor q_lat, Tensor q, int64_t rot_off,
+                                   Tensor cache, Tensor vgroups, Tensor block_tables,
+                                   Tensor seq_lens, Tensor q_start, Tensor tile_seq,
+                                   Tensor tile_row, int64_t tile_rows, double scale) {
+  auto p = latent_mfma_params(out, q_lat, q, rot_off, cache, vgroups, block_tables, seq_lens, scale);
+  CHECK_GPU(q_start); CHECK_GPU(tile_seq); CHECK_GPU(tile_row);
+  CHECK_CONTIG(q_start); CHECK_CONTIG(tile_seq); CHECK_CONTIG(tile_row);
+  TORCH_CHECK(q_start.scalar_type() == at::kInt && tile_seq.scalar_type() == at::kInt &&
+                  tile_row.scalar_type() == at::kInt, "int32 tile map");
+  TORCH_CHECK(q_start.numel() >= p.B + 1 && tile_row.numel() >= tile_seq.numel(), "tile map sizes");
+  TORCH_CHECK(tile_rows >= 32 && tile_rows % 32 == 0, "tiles are whole 32-token pieces");
+  p.q_start = q_start.data_ptr<int32_t>();
+  p.tile_seq = tile_seq.data_ptr<int32_t>();
+  p.tile_row = tile_row.data_ptr<int32_t>();
+  p.num_tiles = tile_seq.numel();
+  p.tile_rows = tile_rows;
+  const c10::DeviceGuard g(q.device());
+  akap_stream::launch_latent_prefill_mfma(p, cur_stream());
+}
+
+void latent_attention_decode_mfma(Tensor out, Tensor q_lat, Tensor q, int64_t rot_off,
+                                  Tensor cache, Tensor vgroups, Tensor block_tables,
+                                  Tensor seq_lens, double scale, std::optional<Tensor> ws_ml,
+                                  std::optional<Tensor> ws_o, int64_t num_parts) {
+  auto p = latent_mfma_params(out, q_lat, q, rot_off, cache, vgroups, block_tables, seq_lens, scale);
+  TORCH_CHECK(p.T == p.B, "decode: one query row per sequence");
+  TORCH_CHECK(num_parts >= 1 && num_parts <= 65535 && p.H <= 65535 * 32, "grid limits");
+  p.num_parts = num_parts;
+  if (num_parts > 1) {
+    TORCH_CHECK(ws_ml.has_value() && ws_o.has_value(), "split decode needs a workspace");
+    CHECK_GPU(*ws_ml); CHECK_GPU(*ws_o); CHECK_F32(*ws_ml); CHECK_F32(*ws_o);
+    CHECK_CONTIG(*ws_ml); CHECK_CONTIG(*ws_o);
+    const int64_t n = (int64_t)p.B * p.H * num_parts;
+    TORCH_CHECK(ws_ml->numel() >= 2 * n && ws_o->numel() >= n * p.R, "decode workspace too small");
+    p.ws_ml = ws_ml->data_ptr<float>();
+    p.ws_o = ws_o->data_ptr<float>();
+  }
+  const c10::DeviceGuard g(q.device());
+  akap_stream::launch_latent_decode_mfma(p, cur_stream());
+}
+
+bool latent_mfma_supported(int64_t R, int64_t r) {
+  return akap_stream::latent_mfma_sizes((int)R, (int)r);
 }
 
 void head_gate(Tensor out, Tensor o, Tensor gate) {
@@ -570,7 +670,14 @@ TORCH_LIBRARY(akap_stream, m) {
         "Tensor positions) -> ()");
   m.def("latent_prep(Tensor proj, Tensor(a!) cq_out, Tensor(b!)? cache, Tensor positions, "
         "Tensor slots, Tensor cos_sin, Tensor q_w, Tensor? kv_w, int q_rank, int kv_rank, "
-        "int rot_dim, int q_off, int kv_off, float eps) -> ()");
+        "int rot_dim, int q_off, int kv_off, float eps, Tensor(c!)? vgroups=None) -> ()");
+  m.def("latent_attention_prefill_mfma(Tensor(a!) out, Tensor q_lat, Tensor q, int rot_off, "
+        "Tensor cache, Tensor vgroups, Tensor block_tables, Tensor seq_lens, Tensor q_start, "
+        "Tensor tile_seq, Tensor tile_row, int tile_rows, float scale) -> ()");
+  m.def("latent_attention_decode_mfma(Tensor(a!) out, Tensor q_lat, Tensor q, int rot_off, "
+        "Tensor cache, Tensor vgroups, Tensor block_tables, Tensor seq_lens, float scale, "
+        "Tensor(b!)? ws_ml, Tensor(c!)? ws_o, int num_parts) -> ()");
+  m.def("latent_mfma_supported(int R, int r) -> bool", &latent_mfma_supported);
   m.def("rotate_heads(Tensor(a!) q, Tensor positions, Tensor cos_sin, int offset) -> ()");
   m.def("latent_attention(Tensor(a!) out, Tensor q_lat, Tensor q, int rot_off, Tensor cache, "
         "Tensor block_tables, Tensor seq_lens, Tensor? q_start, Tensor positions, float scale) "
@@ -590,6 +697,8 @@ TORCH_LIBRARY_IMPL(akap_stream, CUDA, m) {
   m.impl("latent_prep", &latent_prep);
   m.impl("rotate_heads", &rotate_heads);
   m.impl("latent_attention", &latent_attention);
+  m.impl("latent_attention_prefill_mfma", &latent_attention_prefill_mfma);
+  m.impl("latent_attention_decode_mfma", &latent_attention_decode_mfma);
   m.impl("head_gate", &head_gate);
   m.impl("xielu", &xielu);
   m.impl("moe_route", &moe_route);

@@ -27,6 +27,7 @@ residual update, the deferred biases and both norms of the next layer are one ke
 from __future__ import annotations
 
 import dataclasses
+import math
 from typing import Optional
 
 import torch
@@ -104,6 +105,8 @@ class PuputarLM:
         self.vocab_start, self.vocab_end = 0, cfg.vocab_size
         self._tables: dict = {}
         self.state: Optional[torch.Tensor] = None
+        self._ws: Optional[tuple] = None
+        self._seg_map: dict = {}
         self._init_weights(seed)
 
     # ------------------------------------------------------------------ weights
@@ -178,8 +181,9 @@ class PuputarLM:
                (p + "mix.dq", lw.w_in[:m.q_rank], same), (p + "mix.dq.norm", lw.dq_norm, same),
                (p + "mix.uq", lw.w_uq, same),
                # [H D, R] -> [H, D, R] and [H V, R] -> [H, R, V]
-               (p + "mix.uk", lw.w_uk, lambda t: t.reshape(H, D, R)),
-               (p + "mix.uv", lw.w_uv, lambda t: t.reshape(H, V, R).transpose(1, 2)),
+               (p + "mix.uk", lw.w_uk, lambda t: self._want(t, (H * D, R)).reshape(H, D, R)),
+               (p + "mix.uv", lw.w_uv,
+                lambda t: self._want(t, (H * V, R)).reshape(H, V, R).transpose(1, 2)),
                (p + "mix.g", lw.w_in[lw.g_off:lw.g_off + m.gate_rows], same),
                (p + "mix.o", lw.w_out[:, :lw.hv], same)]
         if lw.kv_off >= 0:
@@ -200,6 +204,13 @@ class PuputarLM:
                         (p + f"mlp.e{e}.down", lw.w_down[:, e * F_:(e + 1) * F_], same)]
             out += [(p + "mlp.router", lw.router, same), (p + "mlp.correction", lw.correction, same)]
         return out
+
+    @staticmethod
+    def _want(t: torch.Tensor, shape: tuple) -> torch.Tensor:
+        if tuple(t.shape) != shape:
+            raise ValueError(f"checkpoint shape {tuple(t.shape)} does not fit the config "
+                             f"(wanted {shape})")
+        return t
 
     def _all_names(self):
         same = lambda t: t  # noqa: E731
@@ -250,40 +261,59 @@ class PuputarLM:
         prefill tile map (the latent attention kernel takes its grid from the token rows)."""
         return 1, 128, 0
 
+    def _grouped(self, m: LatentAttentionSpec, block_size: int) -> bool:
+        """Does the layer keep the grouped second copy of its latents (the operand layout of
+        the matrix-core attention kernels: bf16 on the GPU, sizes they are built for)?"""
+        if self.device.type != "cuda" or self.dtype != torch.bfloat16 or block_size % 32:
+            return False
+        sops.load_native(required=True)
+        return bool(torch.ops.akap_stream.latent_mfma_supported(m.kv_rank, m.rot_dim))
+
     def kv_block_bytes(self, block_size: int, kv_dtype: str = "auto") -> int:
         es = torch.empty(0, dtype=self.dtype).element_size()
-        return sum(block_size * self.cfg.layer_specs[i].mixer.cache_dim * es
-                   for i in self.runs if self.cfg.layer_specs[i].mixer.kv_from is None)
-
-    def allocate_kv_segments(self, num_blocks: int, block_size: int, kv_dtype: str = "auto",
-                             max_segment_bytes: Optional[int] = None) -> list:
-        """One allocation [NB, BS, kv_rank + rot_dim] per layer that projects its own latent
-        (zero-filled, the model's dtype): a cached token is ONE row, [latent | rotated key]."""
-        if kv_dtype not in ("auto", "bf16", "bfloat16"):
-            raise ValueError("Puputar: the latent cache is kept in the model's dtype (no fp8)")
-        segs = []
+        n = 0
         for i in self.runs:
             m = self.cfg.layer_specs[i].mixer
             if m.kv_from is None:
-                segs.append(torch.zeros(num_blocks, block_size, m.cache_dim, dtype=self.dtype,
-                                        device=self.device))
+                n += block_size * es * (m.cache_dim + (m.kv_rank if self._grouped(m, block_size)
+                                                       else 0))
+        return n
+
+    def allocate_kv_segments(self, num_blocks: int, block_size: int, kv_dtype: str = "auto",
+                             max_segment_bytes: Optional[int] = None) -> list:
+        """Per layer that projects its own latent: one allocation [NB, BS, kv_rank + rot_dim]
+        (a cached token is ONE row, [latent | rotated key]) and, where the matrix-core kernels
+        run, the latents again as [NB, BS / 8, kv_rank, 8].  Zero-filled, the model's dtype."""
+        if kv_dtype not in ("auto", "bf16", "bfloat16"):
+            raise ValueError("Puputar: the latent cache is kept in the model's dtype (no fp8)")
+        segs, self._seg_map = [], {}
+        for i in self.runs:
+            m = self.cfg.layer_specs[i].mixer
+            if m.kv_from is not None:
+                continue
+            self._seg_map[i] = [len(segs), None]
+            segs.append(torch.zeros(num_blocks, block_size, m.cache_dim, dtype=self.dtype,
+                                    device=self.device))
+            if self._grouped(m, block_size):
+                self._seg_map[i][1] = len(segs)
+                segs.append(torch.zeros(num_blocks, block_size // 8, m.kv_rank, 8,
+                                        dtype=self.dtype, device=self.device))
         return segs
 
     def allocate_kv_cache(self, num_blocks: int, block_size: int, kv_dtype: str = "auto"):
         return self.allocate_kv_segments(num_blocks, block_size, kv_dtype)
 
     def cache_views(self, kv, block_size: int):
-        """Per layer run: its own cache, or the cache of the layer it reads (both lists are the
-        same: keys and values are one row)."""
-        own, segs = {}, list(kv)
-        for i in self.runs:
-            if self.cfg.layer_specs[i].mixer.kv_from is None:
-                own[i] = segs[len(own)]
-        views = []
+        """Per layer run: (row caches, grouped copies or None) of its own latents or of the
+        layer it reads."""
+        segs = list(kv)
+        rows, groups = [], []
         for i in self.runs:
             j = self.cfg.layer_specs[i].mixer.kv_from
-            views.append(own[i if j is None else j])
-        return views, views
+            a, b = self._seg_map[i if j is None else j]
+            rows.append(segs[a])
+            groups.append(segs[b] if b is not None else None)
+        return rows, groups
 
     def allocate_state(self, num_slots: int) -> None:
         """The token shift's previous row per layer run and sequence slot."""
@@ -295,6 +325,48 @@ class PuputarLM:
         if self.dtype == torch.bfloat16:
             return ops.linear(x, w)
         return F.linear(x, w)
+
+    def _decode_parts(self, rows: int, heads: int) -> int:
+        """Key partitions of a decode row: static in the batch size and the model length
+        (hipGraph-capturable), one wave per (row, 32 heads, partition), about 4 waves per CU."""
+        max_parts = max(1, math.ceil(self.max_model_len / 128))
+        waves = max(1, rows * math.ceil(heads / 32))
+        return 1 if waves >= 1024 else min(max_parts, 64, math.ceil(1024 / waves))
+
+    def _workspace(self, rows: int, heads: int, kv_rank: int, parts: int):
+        need = rows * heads * parts * kv_rank
+        if self._ws is None or self._ws[0] < need:
+            # grown on eager steps only: the runner warms every bucket before capturing it
+            self._ws = (need, sops.latent_decode_workspace(rows, heads, kv_rank, parts,
+                                                           self.device))
+        return self._ws[1]
+
+    def _attention(self, m: LatentAttentionSpec, o_lat, q_lat, q, batch: AttnBatch, cache,
+                   groups) -> None:
+        T = q.shape[0]
+        nd = batch.num_decode if batch.is_prefill else T
+        if nd:
+            parts, ws = 1, None
+            if groups is not None:
+                parts = self._decode_parts(nd, m.heads)
+                ws = self._workspace(nd, m.heads, m.kv_rank, parts) if parts > 1 else None
+            # the leading nd rows are contiguous slices of the head-major buffers only when
+            # they are all rows; a mixed step's decode rows go through narrow copies
+            if nd == T:
+                sops.latent_attention_decode(o_lat, q_lat, q, m.dim, cache, groups,
+                                             batch.block_tables[:nd], batch.seq_lens[:nd],
+                                             batch.positions[:nd], m.scale, ws, parts)
+            else:
+                od = torch.empty(m.heads, nd, m.kv_rank, dtype=o_lat.dtype, device=o_lat.device)
+                sops.latent_attention_decode(od, q_lat[:, :nd].contiguous(), q[:nd], m.dim, cache,
+                                             groups, batch.block_tables[:nd], batch.seq_lens[:nd],
+                                             batch.positions[:nd], m.scale, ws, parts)
+                o_lat[:, :nd] = od
+        if batch.is_prefill:
+            sops.latent_attention_prefill(o_lat, q_lat, q, m.dim, cache, groups,
+                                          batch.block_tables, batch.seq_lens, batch.q_start,
+                                          batch.positions, batch.tile_seq, batch.tile_row,
+                                          batch.tile_rows, m.scale, first_seq=nd)
 
     def _routed(self, lw: LatentLayerWeights, h2: torch.Tensor, small: bool) -> torch.Tensor:
         """The routed feed-forward of h2 [T, d] as fp32 [T, d]."""
@@ -347,7 +419,6 @@ class PuputarLM:
         n2 = torch.empty(T, d, dtype=dt, device=dev)
         h = torch.empty(T, d, dtype=dt, device=dev)
         y = y2 = bias = None
-        q_start = batch.q_start if batch.is_prefill else None
         for r, li in enumerate(self.runs):
             lw = self.layers[li]
             m: LatentAttentionSpec = lw.spec.mixer
@@ -359,13 +430,12 @@ class PuputarLM:
             cq = torch.empty(T, m.q_rank, dtype=dt, device=dev)
             sops.latent_prep(proj, cq, k_caches[r] if lw.kv_off >= 0 else None, batch.positions,
                              batch.slots, lw.cos_sin, lw.dq_norm, lw.dkv_norm, m.q_rank, R, rd,
-                             0, lw.kv_off, eps)
+                             0, lw.kv_off, eps, v_caches[r] if lw.kv_off >= 0 else None)
             q = self._linear(cq, lw.w_uq).view(T, H, D + rd)
             sops.rotate_heads_(q, batch.positions, lw.cos_sin, D)
             q_lat = torch.bmm(q[:, :, :D].transpose(0, 1), lw.w_uk)           # [H, T, R]
             o_lat = torch.empty(H, T, R, dtype=dt, device=dev)
-            sops.latent_attention(o_lat, q_lat, q, D, k_caches[r], batch.block_tables,
-                                  batch.seq_lens, q_start, batch.positions, m.scale)
+            self._attention(m, o_lat, q_lat, q, batch, k_caches[r], v_caches[r])
             o = torch.bmm(o_lat, lw.w_uv)                                      # [H, T, V]
             cat = torch.empty(T, lw.hv + lw.ff, dtype=dt, device=dev)
             sops.head_gate(o, proj[:, lw.g_off:lw.g_off + m.gate_rows], cat[:, :lw.hv])

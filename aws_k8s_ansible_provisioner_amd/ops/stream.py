@@ -367,18 +367,21 @@ def _rotate_pairs(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
 def latent_prep(proj: torch.Tensor, cq_out: torch.Tensor, cache: Optional[torch.Tensor],
                 positions: torch.Tensor, slots: torch.Tensor, cos_sin: torch.Tensor,
                 q_w: torch.Tensor, kv_w: Optional[torch.Tensor], q_rank: int, kv_rank: int,
-                rot_dim: int, q_off: int, kv_off: int, eps: float) -> None:
+                rot_dim: int, q_off: int, kv_off: int, eps: float,
+                vgroups: Optional[torch.Tensor] = None) -> None:
     """Per token t of the fused down-projection proj [T, N]: the query latent
     proj[t, q_off : q_off + q_rank] is RMS-normalised (weights q_w, fp32) into cq_out
     [T, q_rank]; the key/value latent proj[t, kv_off : kv_off + kv_rank] is RMS-normalised
     (kv_w) and the next rot_dim entries rotated in interleaved pairs by the angle row of
     positions[t], and both are written as one row [kv_rank + rot_dim] of the paged latent
     cache [NB, BS, kv_rank + rot_dim] at slots[t] (-1: nothing).  cache None: the layer reads
-    another layer's cache and projects no latent of its own."""
+    another layer's cache and projects no latent of its own.  vgroups
+    [NB, BS / 8, kv_rank, 8]: the normed latent once more, in groups of 8 tokens
+    (dimension-major inside a group: the operand layout of the matrix-core attention)."""
     if _native(proj):
         torch.ops.akap_stream.latent_prep(proj, cq_out, cache, positions, slots, cos_sin, q_w,
                                           kv_w, q_rank, kv_rank, rot_dim, q_off, kv_off,
-                                          float(eps))
+                                          float(eps), vgroups)
         return
     cq = _rms(proj[:, q_off:q_off + q_rank].float(), eps) * q_w.float()
     cq_out.copy_(cq.to(cq_out.dtype))
@@ -391,6 +394,8 @@ def latent_prep(proj: torch.Tensor, cq_out: torch.Tensor, cache: Optional[torch.
     ok = slots >= 0
     sl = slots[ok].long()
     cache[sl // BS, sl % BS] = torch.cat([c, kr], dim=1)[ok].to(cache.dtype)
+    if vgroups is not None:
+        vgroups[sl // BS, (sl % BS) // 8, :, sl % 8] = c[ok].to(vgroups.dtype)
 
 
 def rotate_heads_(q: torch.Tensor, positions: torch.Tensor, cos_sin: torch.Tensor,
@@ -440,6 +445,64 @@ def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q: torch.Tensor, ro
         s = (s * scale).masked_fill(~ok[None], float("-inf"))
         out[:, r0:r1] = torch.einsum("htj,jr->htr", torch.softmax(s, dim=-1),
                                      rows[:, :R]).to(out.dtype)
+
+
+def latent_mfma_ok(cache: torch.Tensor, vgroups: Optional[torch.Tensor], kv_rank: int,
+                   q: torch.Tensor, rot_off: int, scale: float) -> bool:
+    """The matrix-core kernels take a bf16 GPU cache with its grouped copy, latent / rotated
+    sizes they were built for, 32-token-aligned blocks and 16-byte-aligned query rows."""
+    if vgroups is None or not cache.is_cuda or cache.dtype != torch.bfloat16:
+        return False
+    load_native(required=True)
+    return (torch.ops.akap_stream.latent_mfma_supported(kv_rank, cache.shape[2] - kv_rank)
+            and cache.shape[1] % 32 == 0 and rot_off % 8 == 0 and q.shape[2] % 8 == 0
+            and scale > 0)
+
+
+def latent_attention_prefill(out: torch.Tensor, q_lat: torch.Tensor, q: torch.Tensor,
+                             rot_off: int, cache: torch.Tensor, vgroups: Optional[torch.Tensor],
+                             block_tables: torch.Tensor, seq_lens: torch.Tensor,
+                             q_start: torch.Tensor, positions: torch.Tensor, tile_seq, tile_row,
+                             tile_rows: int, scale: float, first_seq: int = 0) -> None:
+    """latent_attention for the prompt chunks of a step (sequences from first_seq on; the rows
+    before q_start[first_seq] belong to single-token sequences and are left alone): on the
+    matrix cores when latent_mfma_ok, driven by the scheduler's tile map (tile_seq / tile_row:
+    sequence and first chunk row of a tile of tile_rows tokens), else the row kernel."""
+    if latent_mfma_ok(cache, vgroups, q_lat.shape[2], q, rot_off, scale):
+        torch.ops.akap_stream.latent_attention_prefill_mfma(
+            out, q_lat, q, rot_off, cache, vgroups, block_tables, seq_lens, q_start, tile_seq,
+            tile_row, tile_rows, float(scale))
+        return
+    if first_seq:
+        # the leading rows were handled as decode rows: hide their sequences from this pass
+        seq_lens = seq_lens.clone()
+        seq_lens[:first_seq] = 0
+    latent_attention(out, q_lat, q, rot_off, cache, block_tables, seq_lens, q_start, positions,
+                     scale)
+
+
+def latent_decode_workspace(rows: int, heads: int, kv_rank: int, parts: int, device):
+    n = max(1, rows * heads * parts)
+    return (torch.empty(n * 2, dtype=torch.float32, device=device),
+            torch.empty(n * kv_rank, dtype=torch.float32, device=device))
+
+
+def latent_attention_decode(out: torch.Tensor, q_lat: torch.Tensor, q: torch.Tensor, rot_off: int,
+                            cache: torch.Tensor, vgroups: Optional[torch.Tensor],
+                            block_tables: torch.Tensor, seq_lens: torch.Tensor,
+                            positions: torch.Tensor, scale: float, workspace=None,
+                            num_parts: int = 1) -> None:
+    """latent_attention with one query per sequence, at position seq_lens[b] - 1 (0: a padding
+    row, left unwritten).  On the matrix cores (latent_mfma_ok) the heads of a token are the
+    columns of one tile and the keys are cut into num_parts partitions of whole 32-key blocks,
+    one wave each, merged by a second launch (workspace from latent_decode_workspace)."""
+    if latent_mfma_ok(cache, vgroups, q_lat.shape[2], q, rot_off, scale):
+        ws_ml, ws_o = workspace if (workspace is not None and num_parts > 1) else (None, None)
+        torch.ops.akap_stream.latent_attention_decode_mfma(
+            out, q_lat, q, rot_off, cache, vgroups, block_tables, seq_lens, float(scale), ws_ml,
+            ws_o, num_parts if ws_ml is not None else 1)
+        return
+    latent_attention(out, q_lat, q, rot_off, cache, block_tables, seq_lens, None, positions, scale)
 
 
 def head_gate(o: torch.Tensor, gate: torch.Tensor, out: torch.Tensor) -> None:

@@ -293,3 +293,97 @@ def test_other_configurations(tmp_path, name, dtype):
     sched = [[("p", 17), ("q", 2)], [("p", 1), ("q", 30)], [("p", 27), ("q", 1)],
              [("q", 1)], [("q", 4)]]
     check(replay(eng, reqs, sched), want, dtype)
+
+
+# ------------------------------------------------------------------ matrix-core attention
+def _tile_map(q_start, seq_lens, first_seq, tile_rows):
+    """Tiles of tile_rows chunk rows per sequence, sorted by ascending causal work like the
+    scheduler's map."""
+    tiles = []
+    for b in range(first_seq, len(seq_lens)):
+        qlen = int(q_start[b + 1] - q_start[b])
+        for r0 in range(0, qlen, tile_rows):
+            tiles.append((int(seq_lens[b]) - qlen + min(r0 + tile_rows, qlen), b, r0))
+    tiles.sort()
+    return (torch.tensor([t[1] for t in tiles], dtype=torch.int32),
+            torch.tensor([t[2] for t in tiles], dtype=torch.int32))
+
+
+@pytest.mark.parametrize("H,D,r,R", [(3, 8, 16, 64), (6, 32, 16, 96), (4, 16, 32, 128),
+                                     (33, 8, 32, 256), (16, 128, 64, 512)])
+def test_latent_attention_matrix_core_kernels(H, D, r, R):
+    """Prefill tiles (a chunk that continues a cached prefix, a whole prompt, a short one) and
+    split decode on the matrix cores against the PyTorch op; one far key per sequence is made
+    to matter."""
+    BS, dt = 32, torch.bfloat16
+    lens = [700, 333, 40, 650, 129]
+    chunk = [300, 333, 40]                       # sequences 0..2 bring prompt rows, 3..4 decode
+    T = sum(chunk)
+    cache, bt, rows, w_uk, _, q = _latent_case(R, T, H, D, r, 8, R, BS, lens)
+    for b in range(len(lens)):
+        cache[int(bt[b, 0]), 3] *= 3.0
+    cache = cache.to(dt)
+    vg = sops_groups(cache[..., :R])
+    q_start = torch.tensor([0, 300, 633, 673], dtype=torch.int32)
+    seq_lens = torch.tensor(lens[:3], dtype=torch.int32)
+    pos = torch.cat([torch.arange(n - c, n) for n, c in zip(lens[:3], chunk)])
+    q = (q * 0.5).to(dt)
+    q_lat = (torch.einsum("thd,hdr->htr", q[..., :D].float(), w_uk) * 0.5).to(dt).contiguous()
+    scale = (D + r) ** -0.5
+    want = torch.zeros(H, T, R, dtype=dt)
+    sops.latent_attention(want, q_lat, q, D, cache, bt[:3], seq_lens, q_start, pos, scale)
+    tile_seq, tile_row = _tile_map(q_start, seq_lens, 0, 128)
+    got = torch.zeros(H, T, R, dtype=dt, device="cuda")
+    assert sops.latent_mfma_ok(cache.cuda(), vg.cuda(), R, q.cuda(), D, scale)
+    sops.latent_attention_prefill(got, q_lat.cuda(), q.cuda(), D, cache.cuda(), vg.cuda(),
+                                  bt[:3].cuda(), seq_lens.cuda(), q_start.cuda(), pos.cuda(),
+                                  tile_seq.cuda(), tile_row.cuda(), 128, scale)
+    close(got, want, "bfloat16")
+    # decode rows of sequences 3, 4 and a padding row, unsplit and split
+    seq_d = torch.tensor([650, 129, 0], dtype=torch.int32)
+    btd = torch.cat([bt[3:5], bt[:1]])
+    qd = q[:3].contiguous()
+    qld = q_lat[:, :3].contiguous()
+    posd = torch.tensor([649, 128, 0])
+    want_d = torch.zeros(H, 3, R, dtype=dt)
+    sops.latent_attention(want_d, qld, qd, D, cache, btd, seq_d, None, posd, scale)
+    for parts in (1, 2, 7):
+        got_d = torch.zeros(H, 3, R, dtype=dt, device="cuda")
+        ws = sops.latent_decode_workspace(3, H, R, parts, "cuda")
+        sops.latent_attention_decode(got_d, qld.cuda(), qd.cuda(), D, cache.cuda(), vg.cuda(),
+                                     btd.cuda(), seq_d.cuda(), posd.cuda(), scale, ws, parts)
+        close(got_d, want_d, "bfloat16")
+        assert got_d[:, 2].abs().max().item() == 0
+
+
+def sops_groups(c):
+    """[NB, BS, R] token-major latents in the grouped layout [NB, BS / 8, R, 8]."""
+    NB, BS, R = c.shape
+    return c.view(NB, BS // 8, 8, R).permute(0, 1, 3, 2).contiguous()
+
+
+@pytest.mark.parametrize("eager", [False, True])
+def test_engine_on_the_matrix_core_path(tmp_path, eager):
+    """Sizes the matrix-core kernels take (bf16): prompts over several tiles, portions, mixed
+    steps, a small pool used twice, decoding through hipGraphs with split keys; and the fp32
+    engine of the same model (row kernel) against the oracle, tightly."""
+    cfg = oracle.make_config(width=64, vocab=61, groups=4, layers=[
+        oracle.make_layer(heads=5, dim=16, rot_dim=16, vdim=8, kv_rank=64, q_rank=24),
+        oracle.make_layer(heads=3, dim=8, rot_dim=16, vdim=24, kv_rank=96, q_rank=40,
+                          gate="element", ff=None),
+        oracle.make_layer(heads=6, dim=24, rot_dim=16, vdim=16, kv_rank=64, q_rank=32, kv_from=0,
+                          moe=dict(experts=6, ff=32, top=2, identity=2, count=4, keep=2))])
+    W = oracle.random_weights(cfg, seed=11)
+    reqs = {"a": tokens(390, 61, 1), "b": tokens(200, 61, 2), "c": tokens(35, 61, 3)}
+    want = {n: oracle.forward(cfg, W, t) for n, t in reqs.items()}
+    path = write_model(tmp_path, cfg, W)
+    sched = [[("a", 300), ("b", 2)], [("a", 1), ("b", 150), ("c", 35)], [("a", 1), ("b", 1)],
+             [("a", 60), ("b", 47)], [("a", 28)]]
+    for dtype in ("bfloat16", "float32"):
+        eng = engine(path, dtype=dtype, max_tokens=704, max_seqs=3, device="cuda", eager=eager)
+        grouped = [g is not None for g in eng.runner.v_caches]
+        assert grouped == [dtype == "bfloat16"] * 3
+        for _ in range(2):
+            check(replay(eng, reqs, sched), want, dtype)
+        one = {"a": reqs["a"]}
+        check(replay(eng, one, [[("a", 330)]] + [[("a", 1)]] * 60), want, dtype)
