@@ -262,6 +262,261 @@ __global__ __launch_bounds__(64) void latent_decode_mfma_kernel(LatentAttnParams
       p.ws_o[slot * R + 32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = st.o[dt][i];
 }
 
+
+// ---- wide latents (R >= 256): four waves share one tile of 32 query columns -------------------
+// At R = 512 a single wave's output accumulators alone are 256 registers.  Four waves split the
+// work of a 128-key step instead: wave w scores keys [32 w, 32 w + 32) of the step against the
+// whole query tile (S^T = K Q^T over all R + r dimensions), the waves agree on the running
+// maximum through LDS, publish their bf16 P fragments there, and each wave then accumulates
+// O^T for ITS quarter of the latent dimensions over all 128 keys.  No matrix product is computed
+// twice, a wave holds R / 8 accumulator registers, and two or three workgroups fit a CU.
+template <int NVW>
+struct CoopState {
+  f32x16 o[NVW];   // this wave's quarter of the latent dimensions
+  float m, l;
+};
+
+template <int NV, int NKR>
+struct CoopSmem {
+  static constexpr int DK = 32 * NV + 16 * NKR;
+  static constexpr size_t q_bytes = (size_t)32 * q_pitch(DK) * sizeof(bf16);
+  static constexpr size_t p_bytes = (size_t)4 * 2 * 64 * sizeof(bf16x8);
+  static constexpr size_t bytes = q_bytes + p_bytes + 2 * 4 * 32 * sizeof(float);
+};
+
+template <int NV, int NKR>
+__device__ __forceinline__ void coop_attend(CoopState<NV / 4>& st, const LatentAttnParams& p,
+                                            const int32_t* __restrict__ bt, unsigned char* smem,
+                                            int pos, int pos_min, int jb, int je) {
+  constexpr int R = 32 * NV, DK = R + 16 * NKR, KS = DK / 16, P = q_pitch(DK), NVW = NV / 4;
+  using SM = CoopSmem<NV, NKR>;
+  const float sc2 = p.scale * 1.44269504088896f;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int col = lane & 31, hf = lane >> 5;
+  const int krow = swap23(col);
+  const bf16* cache = (const bf16*)p.cache;
+  const bf16* vg = (const bf16*)p.vgroups;
+  const bf16* qcol = reinterpret_cast<const bf16*>(smem) + col * P + 8 * hf;
+  bf16x8* sm_p = reinterpret_cast<bf16x8*>(smem + SM::q_bytes);          // [4][2][64]
+  float* sm_max = reinterpret_cast<float*>(smem + SM::q_bytes + SM::p_bytes);   // [4][32]
+  float* sm_sum = sm_max + 4 * 32;                                              // [4][32]
+  auto row_of = [&](int j0) -> size_t {
+    const int bi = j0 / p.BS;
+    int blk = bi < p.max_blocks ? bt[bi] : 0;
+    if (blk < 0 || blk >= p.NB) blk = 0;
+    return (size_t)blk * p.BS + (j0 - bi * p.BS);
+  };
+  for (int j0 = jb; j0 <= je; j0 += 128) {
+    const int jw = j0 + 32 * wave;
+    const bool active = jw <= je;                    // (wave-uniform)
+    float sv[16];
+    float bmax = -INFINITY;
+    if (active) {
+      const bf16* kp = cache + (row_of(jw) + krow) * DK + 8 * hf;
+      f32x16 s;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+      for (int c = 0; c < KS; ++c) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + 16 * c);
+        const bf16x8 qf = *reinterpret_cast<const bf16x8*>(qcol + 16 * c);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf, s, 0, 0, 0);
+        // at most 12 K fragments are requested ahead of the products that use them
+        if (c % 12 == 11) __builtin_amdgcn_sched_barrier(0);
+      }
+      if (jw + 31 <= pos_min) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          sv[i] = s[i];
+          bmax = fmaxf(bmax, sv[i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = jw + 16 * (i >> 3) + 8 * hf + (i & 7);
+          sv[i] = key <= pos ? s[i] : -INFINITY;
+          bmax = fmaxf(bmax, sv[i]);
+        }
+      }
+      bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    }
+    if (hf == 0) sm_max[wave * 32 + col] = bmax;
+    __syncthreads();
+    const float bm = fmaxf(fmaxf(sm_max[col], sm_max[32 + col]),
+                           fmaxf(sm_max[64 + col], sm_max[96 + col]));
+    const float mn = fmaxf(st.m, bm * sc2);
+    const float ms = mn == -INFINITY ? 0.f : mn;
+    const float alpha = __builtin_amdgcn_exp2f(st.m - ms);
+    float psum = 0.f;
+    bf16x8 pb[2];
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], sc2, -ms));
+        psum += sv[i];
+      }
+      psum += __shfl_xor(psum, 32, 64);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) pb[i >> 3][i & 7] = (bf16)sv[i];
+      sm_p[(wave * 2 + 0) * 64 + lane] = pb[0];
+      sm_p[(wave * 2 + 1) * 64 + lane] = pb[1];
+    }
+    if (hf == 0) sm_sum[wave * 32 + col] = psum;
+    st.m = mn;
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int dt = 0; dt < NVW; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) st.o[dt][i] *= alpha;
+    }
+    __syncthreads();
+    st.l = st.l * alpha + ((sm_sum[col] + sm_sum[32 + col]) + (sm_sum[64 + col] + sm_sum[96 + col]));
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const int jk = j0 + 32 * kb;
+      if (jk <= je) {                                // (uniform over the workgroup)
+        const bf16x8 p0 = sm_p[(kb * 2 + 0) * 64 + lane];
+        const bf16x8 p1 = sm_p[(kb * 2 + 1) * 64 + lane];
+        const bf16* vp = vg + (((row_of(jk) >> 3) + hf) * R + 32 * (wave * NVW) + col) * 8;
+#pragma unroll
+        for (int dt = 0; dt < NVW; ++dt) {
+          const bf16x8 v0 = *reinterpret_cast<const bf16x8*>(vp + (size_t)(32 * dt) * 8);
+          const bf16x8 v1 = *reinterpret_cast<const bf16x8*>(vp + ((size_t)2 * R + 32 * dt) * 8);
+          st.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, p0, st.o[dt], 0, 0, 0);
+          st.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, st.o[dt], 0, 0, 0);
+        }
+      }
+    }
+  }
+}
+
+// the workgroup's query tile -> LDS: column c is (token tok(c), head head(c))
+template <int NV, int NKR, typename F>
+__device__ __forceinline__ void coop_load_queries(unsigned char* smem, const LatentAttnParams& p,
+                                                  F col_src) {
+  constexpr int R = 32 * NV, DK = R + 16 * NKR, CH = DK / 8, P = q_pitch(DK);
+  bf16* qs = reinterpret_cast<bf16*>(smem);
+  for (int idx = threadIdx.x; idx < 32 * CH; idx += 256) {
+    const int c = idx / CH, ch = idx - c * CH;
+    int t, h;
+    col_src(c, t, h);
+    const bf16* src = ch * 8 < R
+        ? (const bf16*)p.q_lat + ((size_t)h * p.T + t) * R + ch * 8
+        : (const bf16*)p.q + (size_t)t * p.q_stride + (size_t)h * p.q_head + p.rot_off + ch * 8 - R;
+    *reinterpret_cast<bf16x8*>(qs + c * P + ch * 8) = *reinterpret_cast<const bf16x8*>(src);
+  }
+  __syncthreads();
+}
+
+template <int NVW>
+__device__ __forceinline__ void coop_init(CoopState<NVW>& st) {
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < NVW; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) st.o[dt][i] = 0.f;
+}
+
+// Prefill: flat grid over (32-token sub-tile, head) units, one workgroup of 4 waves each
+template <int NV, int NKR>
+__global__ __launch_bounds__(256) void latent_prefill_coop_kernel(LatentAttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int R = 32 * NV, NVW = NV / 4;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int col = lane & 31, hf = lane >> 5;
+  const int sub = p.tile_rows / 32;
+  const int xcd = blockIdx.x & 7, jx = blockIdx.x >> 3;
+  const int unit = (jx / p.H) * 8 + xcd;             // every exit below is workgroup-uniform
+  if (unit >= p.num_tiles * sub) return;
+  const int h = jx % p.H;
+  const int tile = p.num_tiles - 1 - unit / sub;
+  const int si = sub - 1 - unit % sub;
+  const int b = p.tile_seq[tile];
+  if (b < 0 || b >= p.B) return;
+  const int qs0 = p.q_start[b];
+  const int qlen = p.q_start[b + 1] - qs0;
+  const int kv = p.seq_lens[b];
+  const int rend = min(p.tile_row[tile] + p.tile_rows, qlen);
+  const int r0 = p.tile_row[tile] + 32 * si;
+  if (r0 >= rend || kv < qlen) return;
+  coop_load_queries<NV, NKR>(smem, p, [&](int c, int& t, int& hh) {
+    t = qs0 + (r0 + c < rend ? r0 + c : r0);
+    hh = h;
+  });
+  const int r = r0 + col;
+  const bool valid = r < rend;
+  const int t = qs0 + (valid ? r : r0);
+  CoopState<NVW> st;
+  coop_init(st);
+  const int pos_first = kv - qlen + r0;
+  const int pos_last = kv - qlen + min(r0 + 31, rend - 1);
+  coop_attend<NV, NKR>(st, p, p.block_tables + (size_t)b * p.max_blocks, smem, kv - qlen + r,
+                       pos_first, 0, pos_last);
+  if (!valid) return;
+  const float f = st.l > 0.f ? 1.0f / st.l : 0.f;
+  bf16* o = (bf16*)p.out + ((size_t)h * p.T + t) * R + 32 * (wave * NVW);
+#pragma unroll
+  for (int dt = 0; dt < NVW; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; i += 4) {
+      akap::bf16x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (bf16)(st.o[dt][i + e] * f);
+      *reinterpret_cast<akap::bf16x4*>(o + 32 * dt + 8 * (i >> 2) + 4 * hf) = v;
+    }
+}
+
+// Decode: grid (B, ceil(H / 32), parts), one workgroup of 4 waves; columns are heads
+template <int NV, int NKR>
+__global__ __launch_bounds__(256) void latent_decode_coop_kernel(LatentAttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int R = 32 * NV, NVW = NV / 4;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int col = lane & 31, hf = lane >> 5;
+  const int b = blockIdx.x, part = blockIdx.z;
+  const int c0 = blockIdx.y * 32;
+  const int kv = p.seq_lens[b];
+  if (kv <= 0) return;                               // (workgroup-uniform) a padding row
+  const bool valid = c0 + col < p.H;
+  const int h = valid ? c0 + col : c0;
+  const int pos1 = kv - 1;
+  int per = (pos1 + 1 + p.num_parts - 1) / p.num_parts;
+  per = (per + 127) & ~127;
+  const int jb = part * per;
+  const int je = min(pos1, jb + per - 1);
+  CoopState<NVW> st;
+  coop_init(st);
+  if (jb <= je) {                                    // (workgroup-uniform)
+    coop_load_queries<NV, NKR>(smem, p, [&](int c, int& t, int& hh) {
+      t = b;
+      hh = c0 + c < p.H ? c0 + c : c0;
+    });
+    coop_attend<NV, NKR>(st, p, p.block_tables + (size_t)b * p.max_blocks, smem, pos1, pos1, jb, je);
+  }
+  if (!valid) return;
+  if (p.num_parts == 1) {
+    const float f = st.l > 0.f ? 1.0f / st.l : 0.f;
+    bf16* o = (bf16*)p.out + ((size_t)h * p.T + b) * R + 32 * (wave * NVW);
+#pragma unroll
+    for (int dt = 0; dt < NVW; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        o[32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = (bf16)(st.o[dt][i] * f);
+    return;
+  }
+  const size_t slot = ((size_t)b * p.H + h) * p.num_parts + part;
+  if (wave == 0 && hf == 0) {
+    p.ws_ml[slot * 2] = st.m;
+    p.ws_ml[slot * 2 + 1] = st.l;
+  }
+  float* wo = p.ws_o + slot * R + 32 * (wave * NVW);
+#pragma unroll
+  for (int dt = 0; dt < NVW; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) wo[32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = st.o[dt][i];
+}
+
 // grid (B, H): merge the partitions of one (token, head)
 __global__ __launch_bounds__(64) void latent_decode_merge_kernel(LatentAttnParams p) {
   const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -291,6 +546,12 @@ __global__ __launch_bounds__(64) void latent_decode_merge_kernel(LatentAttnParam
 template <int NV, int NKR>
 void launch_prefill(const LatentAttnParams& p, hipStream_t s) {
   constexpr int DK = 32 * NV + 16 * NKR;
+  if constexpr (NV >= 8) {
+    const int units = p.num_tiles * (p.tile_rows / 32);
+    const unsigned grid = (unsigned)((units + 7) / 8 * 8) * p.H;
+    latent_prefill_coop_kernel<NV, NKR><<<grid, 256, CoopSmem<NV, NKR>::bytes, s>>>(p);
+    return;
+  }
   constexpr size_t per_wave = (size_t)32 * q_pitch(DK) * sizeof(bf16);
   const int units = p.num_tiles * (p.tile_rows / 32);
   // as many heads per workgroup as fit 64 KB of LDS
@@ -310,7 +571,10 @@ template <int NV, int NKR>
 void launch_decode(const LatentAttnParams& p, hipStream_t s) {
   constexpr int DK = 32 * NV + 16 * NKR;
   const dim3 grid(p.B, (p.H + 31) / 32, p.num_parts);
-  latent_decode_mfma_kernel<NV, NKR><<<grid, 64, (size_t)32 * q_pitch(DK) * sizeof(bf16), s>>>(p);
+  if constexpr (NV >= 8)
+    latent_decode_coop_kernel<NV, NKR><<<grid, 256, CoopSmem<NV, NKR>::bytes, s>>>(p);
+  else
+    latent_decode_mfma_kernel<NV, NKR><<<grid, 64, (size_t)32 * q_pitch(DK) * sizeof(bf16), s>>>(p);
   if (p.num_parts > 1) latent_decode_merge_kernel<<<dim3(p.B, p.H), 64, 0, s>>>(p);
 }
 

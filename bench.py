@@ -89,7 +89,7 @@ def parse():
                          "kernel table")
     ap.add_argument("--profile-steps", type=int, default=0,
                     help="extra untimed waves run after timing (for rocprofv3 captures)")
-    ap.add_argument("--compare-design", default=None, choices=["bidetar"],
+    ap.add_argument("--compare-design", default=None, choices=["bidetar", "puputar"],
                     help="instead of the serving wave: prefill and decode throughput of this "
                          "design at real layer sizes (random weights) beside the closest "
                          "existing model of equal size; prints one JSON line with the table")
@@ -103,6 +103,9 @@ COMPARE_SETS = {
     # (model of the design, closest existing model of equal size or None)
     "bidetar": [("bidetar-w2048", "llama-w2048"), ("bidetar-w4096", "llama-w4096"),
                 ("bidetar-w1536-d64", None)],
+    # latent attention + token shift beside the framework's other fp32-stream design at the
+    # same width, depth and head count; the routed variant has no equal-size counterpart
+    "puputar": [("puputar-w2048", "bidetar-w2048"), ("puputar-w2048-moe", None)],
 }
 
 

@@ -108,16 +108,18 @@ def test_bench_gpus_n_without_launcher_starts_n_ranks():
     assert res["ranks"] == 2 and res["config"]["parallelism"] == "dp2"
 
 
-def test_bench_compare_design_option():
+@pytest.mark.parametrize("design,models", [("bidetar", "tiny-bidetar,tiny-llama"),
+                                           ("puputar", "tiny-puputar,tiny-bidetar")])
+def test_bench_compare_design_option(design, models):
     """--compare-design prints one JSON line with prefill and decode throughput per model and
     leaves the default output alone."""
-    cmd = [sys.executable, os.path.join(REPO, "bench.py"), "--compare-design", "bidetar",
-           "--compare-models", "tiny-bidetar,tiny-llama", "--device", "cpu", "--steps", "1"]
+    cmd = [sys.executable, os.path.join(REPO, "bench.py"), "--compare-design", design,
+           "--compare-models", models, "--device", "cpu", "--steps", "1"]
     r = subprocess.run(cmd, capture_output=True, text=True, timeout=420, cwd="/tmp")
     assert r.returncode == 0, r.stderr[-3000:]
     lines = [ln for ln in r.stdout.splitlines() if ln.startswith("{")]
     assert len(lines) == 1, r.stdout
     res = json.loads(lines[0])
-    assert res["compare_design"] == "bidetar" and res["data"] == "synthetic"
-    assert [row["model"] for row in res["rows"]] == ["tiny-bidetar", "tiny-llama"]
+    assert res["compare_design"] == design and res["data"] == "synthetic"
+    assert [row["model"] for row in res["rows"]] == models.split(",")
     assert all(row["prefill_tok_s"] > 0 and row["decode_tok_s"] > 0 for row in res["rows"])
