@@ -97,6 +97,30 @@ __global__ __launch_bounds__(256) void token_shift_kernel(T* __restrict__ out,
   }
 }
 
+// every row is a sequence of its own (decode steps): the row's workgroup reads its state and
+// replaces it, one launch
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_single_kernel(T* __restrict__ out,
+                                                                 const T* __restrict__ h,
+                                                                 const float* __restrict__ mu,
+                                                                 T* __restrict__ state,
+                                                                 const int32_t* __restrict__ slot,
+                                                                 const int64_t* __restrict__ pos,
+                                                                 int d) {
+  const int t = blockIdx.x;
+  const T* hr = h + (size_t)t * d;
+  T* st = slot[t] >= 0 ? state + (size_t)slot[t] * d : nullptr;
+  const bool have = st != nullptr && pos[t] > 0;
+  T* o = out + (size_t)t * d;
+  for (int c = threadIdx.x; c < d; c += 256) {
+    const T raw = hr[c];
+    const float v = (float)raw;
+    const float pv = have ? ldf(st + c) : 0.f;
+    stf(o + c, v + (pv - v) * mu[c]);
+    if (st) st[c] = raw;
+  }
+}
+
 // the last row of every sequence in the batch leaves its unshifted h for the next step
 template <typename T>
 __global__ __launch_bounds__(256) void shift_state_kernel(T* __restrict__ state,
@@ -457,8 +481,17 @@ void launch_add_group_norm(void* out1, void* out2, bool out_f32, int out1_stride
 
 void launch_token_shift(void* out, const void* h, const float* mu, void* state,
                         const int32_t* slot, const int64_t* pos, bool f32, int rows, int d,
-                        hipStream_t s) {
+                        bool single, hipStream_t s) {
   if (rows <= 0) return;
+  if (single) {
+    if (f32)
+      token_shift_single_kernel<float><<<rows, 256, 0, s>>>((float*)out, (const float*)h, mu,
+                                                            (float*)state, slot, pos, d);
+    else
+      token_shift_single_kernel<bf16><<<rows, 256, 0, s>>>((bf16*)out, (const bf16*)h, mu,
+                                                           (bf16*)state, slot, pos, d);
+    return;
+  }
   if (f32) {
     token_shift_kernel<float><<<rows, 256, 0, s>>>((float*)out, (const float*)h, mu,
                                                    (const float*)state, slot, pos, d);

@@ -517,10 +517,11 @@ __global__ __launch_bounds__(256) void latent_decode_coop_kernel(LatentAttnParam
     for (int i = 0; i < 16; ++i) wo[32 * dt + 8 * (i >> 2) + 4 * hf + (i & 3)] = st.o[dt][i];
 }
 
-// grid (B, H): merge the partitions of one (token, head)
-__global__ __launch_bounds__(64) void latent_decode_merge_kernel(LatentAttnParams p) {
-  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  if (p.seq_lens[b] <= 0) return;
+// grid (B, H), 128 threads: merge the partitions of one (token, head)
+__global__ __launch_bounds__(128) void latent_decode_merge_kernel(LatentAttnParams p) {
+  extern __shared__ float wts[];                     // [parts] weights of the partitions
+  const int b = blockIdx.x, h = blockIdx.y;
+  if (p.seq_lens[b] <= 0) return;                    // (workgroup-uniform)
   const size_t base = ((size_t)b * p.H + h) * p.num_parts;
   float m = -INFINITY;
   for (int i = 0; i < p.num_parts; ++i)
@@ -528,17 +529,17 @@ __global__ __launch_bounds__(64) void latent_decode_merge_kernel(LatentAttnParam
   float l = 0.f;
   for (int i = 0; i < p.num_parts; ++i) {
     const float li = p.ws_ml[(base + i) * 2 + 1];
-    if (li > 0.f) l += li * __builtin_amdgcn_exp2f(p.ws_ml[(base + i) * 2] - m);
+    const float w = li > 0.f ? __builtin_amdgcn_exp2f(p.ws_ml[(base + i) * 2] - m) : 0.f;
+    l += li * w;
+    if (threadIdx.x == 0) wts[i] = w;
   }
+  __syncthreads();
   const float f = l > 0.f ? 1.0f / l : 0.f;
   bf16* o = (bf16*)p.out + ((size_t)h * p.T + b) * p.R;
-  for (int d = lane; d < p.R; d += 64) {
+  for (int d = threadIdx.x; d < p.R; d += 128) {
     float a = 0.f;
-    for (int i = 0; i < p.num_parts; ++i) {
-      const float li = p.ws_ml[(base + i) * 2 + 1];
-      if (li > 0.f)
-        a += p.ws_o[(base + i) * p.R + d] * __builtin_amdgcn_exp2f(p.ws_ml[(base + i) * 2] - m);
-    }
+    for (int i = 0; i < p.num_parts; ++i)
+      if (wts[i] > 0.f) a += p.ws_o[(base + i) * p.R + d] * wts[i];
     o[d] = (bf16)(a * f);
   }
 }
@@ -575,7 +576,8 @@ void launch_decode(const LatentAttnParams& p, hipStream_t s) {
     latent_decode_coop_kernel<NV, NKR><<<grid, 256, CoopSmem<NV, NKR>::bytes, s>>>(p);
   else
     latent_decode_mfma_kernel<NV, NKR><<<grid, 64, (size_t)32 * q_pitch(DK) * sizeof(bf16), s>>>(p);
-  if (p.num_parts > 1) latent_decode_merge_kernel<<<dim3(p.B, p.H), 64, 0, s>>>(p);
+  if (p.num_parts > 1)
+    latent_decode_merge_kernel<<<dim3(p.B, p.H), 128, p.num_parts * sizeof(float), s>>>(p);
 }
 
 }  // namespace

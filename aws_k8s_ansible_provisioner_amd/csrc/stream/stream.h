@@ -75,10 +75,11 @@ void launch_add_group_norm(void* out1, void* out2, bool out_f32, int out1_stride
                            float* x, const void* y, bool y_f32, int y_stride, const float* y2,
                            const void* bias, const float* w1, const float* w2, int rows, int d,
                            int groups, float eps, hipStream_t s);
-// out[t] = h[t] + (prev - h[t]) * mu; then the last row of each sequence goes to state[slot]
+// out[t] = h[t] + (prev - h[t]) * mu; then the last row of each sequence goes to state[slot].
+// single: every row is a sequence of its own with a distinct slot (one launch instead of two)
 void launch_token_shift(void* out, const void* h, const float* mu, void* state,
                         const int32_t* slot, const int64_t* pos, bool f32, int rows, int d,
-                        hipStream_t s);
+                        bool single, hipStream_t s);
 
 struct LatentPrepParams {
   const void* proj;   // [T, N] fused down-projection rows

@@ -307,7 +307,8 @@ void add_group_norm(Tensor out1, std::optional<Tensor> out2, Tensor x, std::opti
                                      cur_stream());
 }
 
-void token_shift(Tensor out, Tensor h, Tensor mu, Tensor state, Tensor seq_slot, Tensor positions) {
+void token_shift(Tensor out, Tensor h, Tensor mu, Tensor state, Tensor seq_slot, Tensor positions,
+                 bool single) {
   CHECK_GPU(out); CHECK_GPU(h); CHECK_GPU(mu); CHECK_GPU(state); CHECK_GPU(seq_slot);
   CHECK_GPU(positions);
   CHECK_CONTIG(out); CHECK_CONTIG(h); CHECK_CONTIG(mu); CHECK_CONTIG(state); CHECK_CONTIG(seq_slot);
@@ -326,7 +327,7 @@ void token_shift(Tensor out, Tensor h, Tensor mu, Tensor state, Tensor seq_slot,
   akap_stream::launch_token_shift(out.data_ptr(), h.data_ptr(), mu.data_ptr<float>(),
                                   state.data_ptr(), seq_slot.data_ptr<int32_t>(),
                                   positions.data_ptr<int64_t>(), is_f32(h, "h"), (int)T, (int)d,
-                                  cur_stream());
+                                  single, cur_stream());
 }
 
 void latent_prep(Tensor proj, Tensor cq_out, std::optional<Tensor> cache, Tensor positions,
@@ -667,7 +668,7 @@ TORCH_LIBRARY(akap_stream, m) {
   m.def("add_group_norm(Tensor(a!) out1, Tensor(b!)? out2, Tensor(c!) x, Tensor? y, Tensor? y2, "
         "Tensor? bias, Tensor w1, Tensor? w2, int groups, float eps) -> ()");
   m.def("token_shift(Tensor(a!) out, Tensor h, Tensor mu, Tensor(b!) state, Tensor seq_slot, "
-        "Tensor positions) -> ()");
+        "Tensor positions, bool single=False) -> ()");
   m.def("latent_prep(Tensor proj, Tensor(a!) cq_out, Tensor(b!)? cache, Tensor positions, "
         "Tensor slots, Tensor cos_sin, Tensor q_w, Tensor? kv_w, int q_rank, int kv_rank, "
         "int rot_dim, int q_off, int kv_off, float eps, Tensor(c!)? vgroups=None) -> ()");

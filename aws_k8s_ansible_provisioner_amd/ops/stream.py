@@ -324,15 +324,17 @@ def stream_add_group_norm(x: torch.Tensor, y: Optional[torch.Tensor], y2: Option
 
 
 def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, seq_slot: torch.Tensor,
-                positions: torch.Tensor, out: torch.Tensor) -> None:
+                positions: torch.Tensor, out: torch.Tensor, single: bool = False) -> None:
     """out[t] = h[t] + (prev_t - h[t]) * mu, where prev_t is the UNSHIFTED row of the token
     before t in its sequence: row t-1 when that row is the same sequence's previous position
     (equal seq_slot, positions[t-1] + 1 == positions[t]), zeros at position 0, else what an
     earlier step left in state[seq_slot[t]].  Then state[seq_slot[t]] = h[t] for the last row of
     every sequence in the batch.  state [slots, d] (h's type), mu [d] fp32, seq_slot int32
-    (-1: a padding row, no state read or written)."""
+    (-1: a padding row, no state read or written).  single: the caller guarantees that every
+    row is a sequence of its own with a distinct slot (a decode step), which lets the GPU read
+    and replace the state in one launch."""
     if _native(h):
-        torch.ops.akap_stream.token_shift(out, h, mu, state, seq_slot, positions)
+        torch.ops.akap_stream.token_shift(out, h, mu, state, seq_slot, positions, bool(single))
         return
     T = h.shape[0]
     slot, pos = seq_slot.long(), positions.long()

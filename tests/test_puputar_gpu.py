@@ -73,6 +73,16 @@ def test_token_shift_kernel(dtype):
         res.append((out[:7], st))
     close(res[1][0], res[0][0], dtype)
     assert torch.equal(res[1][1].cpu(), res[0][1])
+    # a decode step (every row a sequence of its own): one launch reads and replaces the state
+    slot1 = torch.tensor([2, 0, 3, 1, -1], dtype=torch.int32)
+    pos1 = torch.tensor([5, 0, 9, 4, 0])
+    res = []
+    for dev in ("cpu", "cuda"):
+        st, out = state.clone().to(dev), torch.zeros(5, d, dtype=dt, device=dev)
+        sops.token_shift(h[:5].to(dev), mu.to(dev), st, slot1.to(dev), pos1.to(dev), out, single=True)
+        res.append((out[:4], st))
+    close(res[1][0], res[0][0], dtype)
+    assert torch.equal(res[1][1].cpu(), res[0][1])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
