@@ -460,6 +460,194 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ ou
   }
 }
 
+
+// ------------------------------------------------------------------ 16-byte variants
+// 4 consecutive elements as floats (16 bytes of fp32, 8 of bf16); the launchers check sizes,
+// strides and pointers for that alignment and fall back to the kernels above otherwise
+__device__ __forceinline__ void ld4(float (&v)[4], const float* p) {
+  const akap::f32x4 x = *reinterpret_cast<const akap::f32x4*>(p);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = x[e];
+}
+__device__ __forceinline__ void ld4(float (&v)[4], const bf16* p) {
+  const akap::bf16x4 x = *reinterpret_cast<const akap::bf16x4*>(p);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = (float)x[e];
+}
+__device__ __forceinline__ void st4(float* p, const float (&v)[4]) {
+  akap::f32x4 x;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) x[e] = v[e];
+  *reinterpret_cast<akap::f32x4*>(p) = x;
+}
+__device__ __forceinline__ void st4(bf16* p, const float (&v)[4]) {
+  akap::bf16x4 x;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) x[e] = (bf16)v[e];
+  *reinterpret_cast<akap::bf16x4*>(p) = x;
+}
+
+// the row's group stays in registers between the sum of squares and the scaled writes when it
+// has at most 1024 NR elements: x is read once and written once
+template <typename TY, typename TO, int NR>
+__global__ __launch_bounds__(256) void add_group_norm_vec_kernel(
+    TO* __restrict__ out1, TO* __restrict__ out2, int out1_stride, int out2_stride,
+    float* __restrict__ x, const TY* __restrict__ y, int y_stride, const float* __restrict__ y2,
+    const TY* __restrict__ bias, const float* __restrict__ w1, const float* __restrict__ w2, int d,
+    int groups, float eps) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  float* xr = x + (size_t)row * d;
+  const TY* yr = y ? y + (size_t)row * y_stride : nullptr;
+  const float* y2r = y2 ? y2 + (size_t)row * d : nullptr;
+  TO* o1 = out1 + (size_t)row * out1_stride;
+  TO* o2 = out2 ? out2 + (size_t)row * out2_stride : nullptr;
+  const int gs = d / groups;
+  const bool add = yr || y2r || bias;
+  for (int g = 0; g < groups; ++g) {
+    const int c0 = g * gs;
+    float v[NR][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int c = (i * 256 + threadIdx.x) * 4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[i][e] = 0.f;
+      if (c < gs) {
+        ld4(v[i], xr + c0 + c);
+        if (add) {
+          float a[4];
+          if (yr) {
+            ld4(a, yr + c0 + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[i][e] += a[e];
+          }
+          if (bias) {
+            ld4(a, bias + c0 + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[i][e] += a[e];
+          }
+          if (y2r) {
+            ld4(a, y2r + c0 + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[i][e] += a[e];
+          }
+          st4(xr + c0 + c, v[i]);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ss += v[i][e] * v[i][e];
+      }
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int c = (i * 256 + threadIdx.x) * 4;
+      if (c < gs) {
+        float w[4], r[4];
+        ld4(w, w1 + c0 + c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = v[i][e] * inv * w[e];
+        st4(o1 + c0 + c, r);
+        if (o2) {
+          ld4(w, w2 + c0 + c);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) r[e] = v[i][e] * inv * w[e];
+          st4(o2 + c0 + c, r);
+        }
+      }
+    }
+  }
+}
+
+// grid (rows, pieces of 4096 columns): a thread takes 4 pieces of 4 columns, 1024 apart
+template <typename T>
+__global__ __launch_bounds__(256) void xielu_vec_kernel(T* __restrict__ out, int out_stride,
+                                                        const T* __restrict__ x, int x_stride,
+                                                        const T* __restrict__ bias,
+                                                        const float* __restrict__ act, int F) {
+  const int t = blockIdx.x;
+  const float ap = softplusf(act[0]), aq = 0.5f + softplusf(act[1]);
+  const T* xr = x + (size_t)t * x_stride;
+  T* o = out + (size_t)t * out_stride;
+  float z[4][4], b[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = blockIdx.y * 4096 + i * 1024 + threadIdx.x * 4;
+    if (c < F) {
+      ld4(z[i], xr + c);
+      if (bias) ld4(b[i], bias + c);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = blockIdx.y * 4096 + i * 1024 + threadIdx.x * 4;
+    if (c < F) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float u = z[i][e] + (bias ? b[i][e] : 0.f);
+        z[i][e] = u > 0.f ? ap * u * u + 0.5f * u : aq * (expm1f(u) - u) + 0.5f * u;
+      }
+      st4(o + c, z[i]);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_vec_kernel(T* __restrict__ out,
+                                                              const T* __restrict__ h,
+                                                              const float* __restrict__ mu,
+                                                              T* __restrict__ state,
+                                                              const int32_t* __restrict__ slot,
+                                                              const int64_t* __restrict__ pos,
+                                                              int d, int single) {
+  const int t = blockIdx.x;
+  const T* hr = h + (size_t)t * d;
+  const T* prev = nullptr;
+  if (!single && continues(slot, pos, t)) prev = hr - d;
+  else if (slot[t] >= 0 && pos[t] > 0) prev = state + (size_t)slot[t] * d;
+  T* st = single && slot[t] >= 0 ? state + (size_t)slot[t] * d : nullptr;
+  T* o = out + (size_t)t * d;
+  for (int c = threadIdx.x * 4; c < d; c += 1024) {
+    float v[4], pv[4] = {0.f, 0.f, 0.f, 0.f}, m[4], r[4];
+    ld4(v, hr + c);
+    if (prev) ld4(pv, prev + c);
+    ld4(m, mu + c);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = v[e] + (pv[e] - v[e]) * m[e];
+    st4(o + c, r);
+    if (st) st4(st + c, v);       // v came from T: the round trip is exact
+  }
+}
+
+// per-head gates, V % 4 == 0: 4 consecutive output entries share a head
+template <typename T>
+__global__ __launch_bounds__(256) void head_gate_vec_kernel(T* __restrict__ out, int out_stride,
+                                                            const T* __restrict__ o,
+                                                            const T* __restrict__ gate,
+                                                            int gate_stride, int per_head, int H,
+                                                            int V, int rows) {
+  const int t = blockIdx.x;
+  const T* g = gate + (size_t)t * gate_stride;
+  T* dst = out + (size_t)t * out_stride;
+  for (int c = threadIdx.x * 4; c < H * V; c += 1024) {
+    const int h = c / V, j = c - h * V;
+    float v[4], z[4];
+    ld4(v, o + ((size_t)h * rows + t) * V + j);
+    if (per_head) {
+      const float zh = ldf(g + h);
+      z[0] = z[1] = z[2] = z[3] = zh;
+    } else {
+      ld4(z, g + c);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] *= sigmoidf(z[e]);
+    st4(dst + c, v);
+  }
+}
+
+bool al(const void* p, size_t a) { return p == nullptr || ((uintptr_t)p % a) == 0; }
+
 }  // namespace
 
 // ------------------------------------------------------------------ launchers
@@ -468,6 +656,28 @@ void launch_add_group_norm(void* out1, void* out2, bool out_f32, int out1_stride
                            const void* bias, const float* w1, const float* w2, int rows, int d,
                            int groups, float eps, hipStream_t s) {
   if (rows <= 0) return;
+  // 16-byte path: every group a multiple of 4 columns that fits 4096 columns in registers
+  const int gsz = d / groups;
+  const size_t ob = out_f32 ? 16 : 8, yb = y_f32 ? 16 : 8;
+  if (gsz % 4 == 0 && gsz <= 4096 && out1_stride % 4 == 0 && out2_stride % 4 == 0 &&
+      y_stride % 4 == 0 && al(x, 16) && al(y2, 16) && al(w1, 16) && al(w2, 16) && al(out1, ob) &&
+      al(out2, ob) && al(y, yb) && al(bias, yb)) {
+#define AGNV(TY, TO, NR)                                                                         \
+  add_group_norm_vec_kernel<TY, TO, NR><<<rows, 256, 0, s>>>(                                    \
+      (TO*)out1, (TO*)out2, out1_stride, out2_stride, x, (const TY*)y, y_stride, y2,             \
+      (const TY*)bias, w1, w2, d, groups, eps)
+#define AGNT(NR)                                                                                 \
+  if (y_f32 && out_f32) AGNV(float, float, NR);                                                  \
+  else if (!y_f32 && out_f32) AGNV(bf16, float, NR);                                             \
+  else if (y_f32) AGNV(float, bf16, NR);                                                         \
+  else AGNV(bf16, bf16, NR)
+    if (gsz <= 1024) { AGNT(1); }
+    else if (gsz <= 2048) { AGNT(2); }
+    else { AGNT(4); }
+#undef AGNT
+#undef AGNV
+    return;
+  }
 #define AGN(TY, TO)                                                                              \
   add_group_norm_kernel<TY, TO><<<rows, 256, 0, s>>>((TO*)out1, (TO*)out2, out1_stride,          \
                                                      out2_stride, x, (const TY*)y, y_stride, y2, \
@@ -483,6 +693,23 @@ void launch_token_shift(void* out, const void* h, const float* mu, void* state,
                         const int32_t* slot, const int64_t* pos, bool f32, int rows, int d,
                         bool single, hipStream_t s) {
   if (rows <= 0) return;
+  const size_t eb = f32 ? 16 : 8;
+  if (d % 4 == 0 && al(out, eb) && al(h, eb) && al(state, eb) && al(mu, 16)) {
+    if (f32) {
+      token_shift_vec_kernel<float><<<rows, 256, 0, s>>>((float*)out, (const float*)h, mu,
+                                                         (float*)state, slot, pos, d, single);
+      if (!single)
+        shift_state_kernel<float><<<rows, 256, 0, s>>>((float*)state, (const float*)h, slot, pos,
+                                                       d, rows);
+    } else {
+      token_shift_vec_kernel<bf16><<<rows, 256, 0, s>>>((bf16*)out, (const bf16*)h, mu,
+                                                        (bf16*)state, slot, pos, d, single);
+      if (!single)
+        shift_state_kernel<bf16><<<rows, 256, 0, s>>>((bf16*)state, (const bf16*)h, slot, pos, d,
+                                                      rows);
+    }
+    return;
+  }
   if (single) {
     if (f32)
       token_shift_single_kernel<float><<<rows, 256, 0, s>>>((float*)out, (const float*)h, mu,
@@ -546,6 +773,19 @@ void launch_latent_attention(const LatentAttnParams& p, bool f32, hipStream_t s)
 void launch_head_gate(void* out, int out_stride, const void* o, const void* gate, int gate_stride,
                       bool per_head, int rows, int H, int V, bool f32, hipStream_t s) {
   if (rows <= 0) return;
+  const size_t eb = f32 ? 16 : 8;
+  if (V % 4 == 0 && out_stride % 4 == 0 && al(out, eb) && al(o, eb) &&
+      (per_head || (gate_stride % 4 == 0 && al(gate, eb)))) {
+    if (f32)
+      head_gate_vec_kernel<float><<<rows, 256, 0, s>>>((float*)out, out_stride, (const float*)o,
+                                                       (const float*)gate, gate_stride, per_head,
+                                                       H, V, rows);
+    else
+      head_gate_vec_kernel<bf16><<<rows, 256, 0, s>>>((bf16*)out, out_stride, (const bf16*)o,
+                                                      (const bf16*)gate, gate_stride, per_head, H,
+                                                      V, rows);
+    return;
+  }
   if (f32)
     head_gate_kernel<float><<<rows, 256, 0, s>>>((float*)out, out_stride, (const float*)o,
                                                  (const float*)gate, gate_stride, per_head, H, V,
@@ -559,6 +799,18 @@ void launch_head_gate(void* out, int out_stride, const void* o, const void* gate
 void launch_xielu(void* out, int out_stride, const void* x, int x_stride, const void* bias,
                   const float* act, int rows, int F, bool f32, hipStream_t s) {
   if (rows <= 0) return;
+  const size_t eb = f32 ? 16 : 8;
+  if (F % 4 == 0 && out_stride % 4 == 0 && x_stride % 4 == 0 && al(out, eb) && al(x, eb) &&
+      al(bias, eb) && (F + 4095) / 4096 <= 65535) {
+    const dim3 grid(rows, (F + 4095) / 4096);
+    if (f32)
+      xielu_vec_kernel<float><<<grid, 256, 0, s>>>((float*)out, out_stride, (const float*)x,
+                                                   x_stride, (const float*)bias, act, F);
+    else
+      xielu_vec_kernel<bf16><<<grid, 256, 0, s>>>((bf16*)out, out_stride, (const bf16*)x, x_stride,
+                                                  (const bf16*)bias, act, F);
+    return;
+  }
   if (f32)
     xielu_kernel<float><<<rows, 256, 0, s>>>((float*)out, out_stride, (const float*)x, x_stride,
                                              (const float*)bias, act, F);

@@ -26,12 +26,14 @@ def close(a, b, dtype):
 
 # ------------------------------------------------------------------ kernels against their ops
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("d,groups", [(24, 4), (2048, 1), (1536, 3), (54, 9), (4100, 2)])
+@pytest.mark.parametrize("d,groups", [(24, 4), (2048, 1), (1536, 3), (54, 9), (4100, 2), (4096, 1),
+                                      (8192, 1), (8192, 4), (40, 2)])
 def test_add_group_norm_kernel(dtype, d, groups):
     g, dt = gen(d), DT[dtype]
     T = 7
     x = torch.randn(T, d, generator=g)
-    y, b = torch.randn(T, d + 3, generator=g).to(dt), torch.randn(d, generator=g).to(dt)
+    # y is a column slice of wider rows (16-byte aligned rows when d allows: the vector path)
+    y, b = torch.randn(T, d + 4, generator=g).to(dt), torch.randn(d, generator=g).to(dt)
     y2 = torch.randn(T, d, generator=g)
     w1, w2 = 1 + 0.3 * torch.randn(d, generator=g), 1 + 0.3 * torch.randn(d, generator=g)
     for use in [(True, True, True, True), (True, False, False, False), (False, False, False, False),
@@ -58,9 +60,9 @@ def test_add_group_norm_kernel(dtype, d, groups):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_token_shift_kernel(dtype):
+@pytest.mark.parametrize("d", [70, 72, 2048])
+def test_token_shift_kernel(dtype, d):
     g, dt = gen(1), DT[dtype]
-    d = 70
     h = torch.randn(9, d, generator=g).to(dt)
     mu = torch.rand(d, generator=g)
     state = torch.randn(4, d, generator=g).to(dt)
@@ -145,12 +147,13 @@ def test_latent_attention_kernel(dtype, H, D, r, V, R):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_gate_activation_and_routing_kernels(dtype):
+@pytest.mark.parametrize("V,F_", [(5, 37), (8, 40), (128, 2052)])
+def test_gate_activation_and_routing_kernels(dtype, V, F_):
     g, dt = gen(4), DT[dtype]
-    H, T, V, F_ = 3, 6, 5, 37
+    H, T = 3, 6
     o = torch.randn(H, T, V, generator=g).to(dt)
-    wide = torch.randn(T, 2 + H * V + 1, generator=g).to(dt)
-    x = (torch.randn(T, F_ + 2, generator=g) * 3).to(dt)
+    wide = torch.randn(T, 4 + H * V + 4, generator=g).to(dt)
+    x = (torch.randn(T, F_ + 8, generator=g) * 3).to(dt)
     b = torch.randn(F_, generator=g).to(dt)
     act = torch.tensor([-0.7, 1.3])
     n, d, E = 12, 40, 9
@@ -162,11 +165,11 @@ def test_gate_activation_and_routing_kernels(dtype):
     for dev in ("cpu", "cuda"):
         r = []
         for cols in (H, H * V):
-            out = torch.zeros(T, H * V + 3, dtype=dt, device=dev)
-            sops.head_gate(o.to(dev), wide[:, 2:2 + cols].to(dev), out[:, :H * V])
+            out = torch.zeros(T, H * V + 4, dtype=dt, device=dev)
+            sops.head_gate(o.to(dev), wide.to(dev)[:, 4:4 + cols], out[:, :H * V])
             r.append(out)
-        out = torch.zeros(T, F_ + 1, dtype=dt, device=dev)
-        sops.xielu(x[:, 1:1 + F_].to(dev), b.to(dev), act.to(dev), out[:, :F_])
+        out = torch.zeros(T, F_ + 4, dtype=dt, device=dev)
+        sops.xielu(x.to(dev)[:, 4:4 + F_], b.to(dev), act.to(dev), out[:, :F_])
         r.append(out)
         for count, keep, top in [(1, 1, 4), (3, 2, 4), (4, 1, 3), (12, 5, 4)]:
             ids, w = sops.moe_route(h.to(dev), router.to(dev), corr.to(dev), top, count, keep)
