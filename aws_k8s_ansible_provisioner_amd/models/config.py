@@ -562,6 +562,9 @@ PUPUTAR_W2048 = register(_puputar_stack(
 PUPUTAR_W2048_MOE = register(_puputar_stack(
     "puputar-w2048-moe", width=2048, n=16, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512,
     q_rank=768, ff=8192, experts=14, expert_ff=2048, top=4, identity=2, groups=4, keep=2))
+PUPUTAR_W4096 = register(_puputar_stack(
+    "puputar-w4096", width=4096, n=8, heads=32, dim=128, rot_dim=64, vdim=128, kv_rank=512,
+    q_rank=1536, ff=21504, norm_groups=4))
 TINY_PUPUTAR = register(_puputar_stack(
     "tiny-puputar", width=128, n=6, heads=4, dim=16, rot_dim=8, vdim=24, kv_rank=40, q_rank=48,
     ff=192, experts=6, expert_ff=64, top=3, identity=2, groups=4, keep=2, vocab=512,

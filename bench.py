@@ -105,7 +105,8 @@ COMPARE_SETS = {
                 ("bidetar-w1536-d64", None)],
     # latent attention + token shift beside the framework's other fp32-stream design at the
     # same width, depth and head count; the routed variant has no equal-size counterpart
-    "puputar": [("puputar-w2048", "bidetar-w2048"), ("puputar-w2048-moe", None)],
+    "puputar": [("puputar-w2048", "bidetar-w2048"), ("puputar-w4096", "bidetar-w4096"),
+                ("puputar-w2048-moe", None)],
 }
 
 
