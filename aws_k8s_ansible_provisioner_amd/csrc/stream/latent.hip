@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void add_group_norm_kernel(
     TO* __restrict__ out1, TO* __restrict__ out2, int out1_stride, int out2_stride,
     float* __restrict__ x, const TY* __restrict__ y, int y_stride, const float* __restrict__ y2,
     const TY* __restrict__ bias, const float* __restrict__ w1, const float* __restrict__ w2, int d,
-    int groups, float eps) {
+    int groups, float eps, ShiftArgs sh) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   float* xr = x + (size_t)row * d;
@@ -45,6 +45,9 @@ __global__ __launch_bounds__(256) void add_group_norm_kernel(
   TO* o2 = out2 ? out2 + (size_t)row * out2_stride : nullptr;
   const int gs = d / groups;
   const bool add = yr || y2r || bias;
+  // token shift of out1 for rows that are sequences of their own (see ShiftArgs)
+  TO* st = sh.mu && sh.slot[row] >= 0 ? (TO*)sh.state + (size_t)sh.slot[row] * d : nullptr;
+  const bool have = st != nullptr && sh.pos[row] > 0;
   for (int g = 0; g < groups; ++g) {
     const int c0 = g * gs, c1 = c0 + gs;
     float ss = 0.f;
@@ -66,7 +69,14 @@ __global__ __launch_bounds__(256) void add_group_norm_kernel(
     // each thread re-reads the columns it wrote itself
     for (int c = c0 + threadIdx.x; c < c1; c += 256) {
       const float n = xr[c] * inv;
-      stf(o1 + c, n * w1[c]);
+      if (sh.mu) {
+        const TO h = (TO)(n * w1[c]);                // the unshifted row, as stored
+        const float hv = (float)h, pv = have ? ldf(st + c) : 0.f;
+        stf(o1 + c, hv + (pv - hv) * sh.mu[c]);
+        if (st) st[c] = h;
+      } else {
+        stf(o1 + c, n * w1[c]);
+      }
       if (o2) stf(o2 + c, n * w2[c]);
     }
   }
@@ -494,7 +504,7 @@ __global__ __launch_bounds__(256) void add_group_norm_vec_kernel(
     TO* __restrict__ out1, TO* __restrict__ out2, int out1_stride, int out2_stride,
     float* __restrict__ x, const TY* __restrict__ y, int y_stride, const float* __restrict__ y2,
     const TY* __restrict__ bias, const float* __restrict__ w1, const float* __restrict__ w2, int d,
-    int groups, float eps) {
+    int groups, float eps, ShiftArgs sh) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   float* xr = x + (size_t)row * d;
@@ -504,6 +514,8 @@ __global__ __launch_bounds__(256) void add_group_norm_vec_kernel(
   TO* o2 = out2 ? out2 + (size_t)row * out2_stride : nullptr;
   const int gs = d / groups;
   const bool add = yr || y2r || bias;
+  TO* st = sh.mu && sh.slot[row] >= 0 ? (TO*)sh.state + (size_t)sh.slot[row] * d : nullptr;
+  const bool have = st != nullptr && sh.pos[row] > 0;
   for (int g = 0; g < groups; ++g) {
     const int c0 = g * gs;
     float v[NR][4];
@@ -548,6 +560,16 @@ __global__ __launch_bounds__(256) void add_group_norm_vec_kernel(
         ld4(w, w1 + c0 + c);
 #pragma unroll
         for (int e = 0; e < 4; ++e) r[e] = v[i][e] * inv * w[e];
+        if (sh.mu) {
+          float pv[4] = {0.f, 0.f, 0.f, 0.f}, m[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) r[e] = (float)(TO)r[e];   // the unshifted row, as stored
+          if (have) ld4(pv, st + c0 + c);
+          ld4(m, sh.mu + c0 + c);
+          if (st) st4(st + c0 + c, r);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) r[e] = r[e] + (pv[e] - r[e]) * m[e];
+        }
         st4(o1 + c0 + c, r);
         if (o2) {
           ld4(w, w2 + c0 + c);
@@ -654,18 +676,18 @@ bool al(const void* p, size_t a) { return p == nullptr || ((uintptr_t)p % a) == 
 void launch_add_group_norm(void* out1, void* out2, bool out_f32, int out1_stride, int out2_stride,
                            float* x, const void* y, bool y_f32, int y_stride, const float* y2,
                            const void* bias, const float* w1, const float* w2, int rows, int d,
-                           int groups, float eps, hipStream_t s) {
+                           int groups, float eps, const ShiftArgs& sh, hipStream_t s) {
   if (rows <= 0) return;
   // 16-byte path: every group a multiple of 4 columns that fits 4096 columns in registers
   const int gsz = d / groups;
   const size_t ob = out_f32 ? 16 : 8, yb = y_f32 ? 16 : 8;
   if (gsz % 4 == 0 && gsz <= 4096 && out1_stride % 4 == 0 && out2_stride % 4 == 0 &&
       y_stride % 4 == 0 && al(x, 16) && al(y2, 16) && al(w1, 16) && al(w2, 16) && al(out1, ob) &&
-      al(out2, ob) && al(y, yb) && al(bias, yb)) {
+      al(out2, ob) && al(y, yb) && al(bias, yb) && al(sh.mu, 16) && al(sh.state, ob)) {
 #define AGNV(TY, TO, NR)                                                                         \
   add_group_norm_vec_kernel<TY, TO, NR><<<rows, 256, 0, s>>>(                                    \
       (TO*)out1, (TO*)out2, out1_stride, out2_stride, x, (const TY*)y, y_stride, y2,             \
-      (const TY*)bias, w1, w2, d, groups, eps)
+      (const TY*)bias, w1, w2, d, groups, eps, sh)
 #define AGNT(NR)                                                                                 \
   if (y_f32 && out_f32) AGNV(float, float, NR);                                                  \
   else if (!y_f32 && out_f32) AGNV(bf16, float, NR);                                             \
@@ -681,7 +703,7 @@ void launch_add_group_norm(void* out1, void* out2, bool out_f32, int out1_stride
 #define AGN(TY, TO)                                                                              \
   add_group_norm_kernel<TY, TO><<<rows, 256, 0, s>>>((TO*)out1, (TO*)out2, out1_stride,          \
                                                      out2_stride, x, (const TY*)y, y_stride, y2, \
-                                                     (const TY*)bias, w1, w2, d, groups, eps)
+                                                     (const TY*)bias, w1, w2, d, groups, eps, sh)
   if (y_f32 && out_f32) AGN(float, float);
   else if (!y_f32 && out_f32) AGN(bf16, float);
   else if (y_f32) AGN(float, bf16);

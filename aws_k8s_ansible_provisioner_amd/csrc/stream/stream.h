@@ -71,10 +71,19 @@ void launch_sink_attention_decode(const AttnParams& p, bool f32, hipStream_t s);
 // x (fp32 rows of d) += y + bias + y2 (each may be null; y / bias of the activation type, y2
 // fp32), then out1 = gnorm(x) * w1 and out2 = gnorm(x) * w2 (out2 / w2 may be null), the norm
 // taken over `groups` equal consecutive parts of the row
+// optional token shift of out1 inside the norm kernel, for batches whose every row is a sequence
+// of its own with a distinct slot (decode steps): out1 = h + (state[slot] - h) * mu with h the
+// normed row as stored (zeros for position 0), and state[slot] = h.  mu null: no shift.
+struct ShiftArgs {
+  const float* mu;       // [d]
+  void* state;           // [slots, d] of out1's type
+  const int32_t* slot;   // [rows]
+  const int64_t* pos;    // [rows]
+};
 void launch_add_group_norm(void* out1, void* out2, bool out_f32, int out1_stride, int out2_stride,
                            float* x, const void* y, bool y_f32, int y_stride, const float* y2,
                            const void* bias, const float* w1, const float* w2, int rows, int d,
-                           int groups, float eps, hipStream_t s);
+                           int groups, float eps, const ShiftArgs& sh, hipStream_t s);
 // out[t] = h[t] + (prev - h[t]) * mu; then the last row of each sequence goes to state[slot].
 // single: every row is a sequence of its own with a distinct slot (one launch instead of two)
 void launch_token_shift(void* out, const void* h, const float* mu, void* state,

@@ -251,7 +251,9 @@ void sink_attention_decode(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
 // ---- grouped norms, token shift, latent attention, routed experts ----------------------------
 void add_group_norm(Tensor out1, std::optional<Tensor> out2, Tensor x, std::optional<Tensor> y,
                     std::optional<Tensor> y2, std::optional<Tensor> bias, Tensor w1,
-                    std::optional<Tensor> w2, int64_t groups, double eps) {
+                    std::optional<Tensor> w2, int64_t groups, double eps,
+                    std::optional<Tensor> shift_mu, std::optional<Tensor> shift_state,
+                    std::optional<Tensor> seq_slot, std::optional<Tensor> positions) {
   CHECK_GPU(out1); CHECK_GPU(x); CHECK_GPU(w1);
   CHECK_F32(x); CHECK_CONTIG(x); CHECK_F32(w1); CHECK_CONTIG(w1); CHECK_LAST_CONTIG(out1);
   TORCH_CHECK(x.dim() == 2 && out1.dim() == 2 && out1.sizes() == x.sizes(),
@@ -300,11 +302,28 @@ void add_group_norm(Tensor out1, std::optional<Tensor> out2, Tensor x, std::opti
     TORCH_CHECK(y2->sizes() == x.sizes(), "add_group_norm: y2 shape");
     y2p = y2->data_ptr<float>();
   }
+  akap_stream::ShiftArgs sh{};
+  if (shift_mu.has_value()) {
+    TORCH_CHECK(shift_state.has_value() && seq_slot.has_value() && positions.has_value(),
+                "add_group_norm: the shift needs state, slots and positions");
+    CHECK_GPU(*shift_mu); CHECK_F32(*shift_mu); CHECK_CONTIG(*shift_mu);
+    CHECK_GPU(*shift_state); CHECK_CONTIG(*shift_state); CHECK_GPU(*seq_slot); CHECK_CONTIG(*seq_slot);
+    CHECK_GPU(*positions); CHECK_CONTIG(*positions);
+    TORCH_CHECK(shift_mu->numel() == d && shift_state->dim() == 2 && shift_state->size(1) == d &&
+                    shift_state->scalar_type() == out1.scalar_type(), "add_group_norm: shift shapes");
+    TORCH_CHECK(seq_slot->scalar_type() == at::kInt && positions->scalar_type() == at::kLong &&
+                    seq_slot->numel() >= rows && positions->numel() >= rows,
+                "add_group_norm: seq_slot int32 / positions int64 per row");
+    sh.mu = shift_mu->data_ptr<float>();
+    sh.state = shift_state->data_ptr();
+    sh.slot = seq_slot->data_ptr<int32_t>();
+    sh.pos = positions->data_ptr<int64_t>();
+  }
   const c10::DeviceGuard g(x.device());
   akap_stream::launch_add_group_norm(out1.data_ptr(), o2, of, (int)out1.stride(0), o2s,
                                      x.data_ptr<float>(), yp, yf, ys, y2p, bp,
                                      w1.data_ptr<float>(), w2p, rows, d, (int)groups, (float)eps,
-                                     cur_stream());
+                                     sh, cur_stream());
 }
 
 void token_shift(Tensor out, Tensor h, Tensor mu, Tensor state, Tensor seq_slot, Tensor positions,
@@ -666,7 +685,8 @@ TORCH_LIBRARY(akap_stream, m) {
       "Tensor block_tables, Tensor seq_lens, Tensor? gate, Tensor? sink, float scale, int chunk, "
       "int window, Tensor(b!)? ws_ml, Tensor(c!)? ws_o, int num_parts) -> ()");
   m.def("add_group_norm(Tensor(a!) out1, Tensor(b!)? out2, Tensor(c!) x, Tensor? y, Tensor? y2, "
-        "Tensor? bias, Tensor w1, Tensor? w2, int groups, float eps) -> ()");
+        "Tensor? bias, Tensor w1, Tensor? w2, int groups, float eps, Tensor? shift_mu=None, "
+        "Tensor(d!)? shift_state=None, Tensor? seq_slot=None, Tensor? positions=None) -> ()");
   m.def("token_shift(Tensor(a!) out, Tensor h, Tensor mu, Tensor(b!) state, Tensor seq_slot, "
         "Tensor positions, bool single=False) -> ()");
   m.def("latent_prep(Tensor proj, Tensor(a!) cq_out, Tensor(b!)? cache, Tensor positions, "

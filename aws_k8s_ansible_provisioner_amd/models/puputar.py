@@ -423,10 +423,16 @@ class PuputarLM:
             lw = self.layers[li]
             m: LatentAttentionSpec = lw.spec.mixer
             H, D, rd, V, R = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
-            sops.stream_add_group_norm(x, y, y2, bias, lw.norm1, lw.norm2, groups, eps, n1,
-                                       n2 if lw.norm2 is not None else None)
-            sops.token_shift(n1, lw.shift, self.state[r], seq_slot, batch.positions, h,
-                             single=not batch.is_prefill)
+            if batch.is_prefill:
+                sops.stream_add_group_norm(x, y, y2, bias, lw.norm1, lw.norm2, groups, eps, n1,
+                                           n2 if lw.norm2 is not None else None)
+                sops.token_shift(n1, lw.shift, self.state[r], seq_slot, batch.positions, h)
+            else:
+                # every row is a sequence of its own: the shift rides in the norm kernel
+                sops.stream_add_group_norm(x, y, y2, bias, lw.norm1, lw.norm2, groups, eps, h,
+                                           n2 if lw.norm2 is not None else None,
+                                           shift=(lw.shift, self.state[r], seq_slot,
+                                                  batch.positions))
             proj = self._linear(h, lw.w_in)                      # [T, dq | dkv | g]
             cq = torch.empty(T, m.q_rank, dtype=dt, device=dev)
             sops.latent_prep(proj, cq, k_caches[r] if lw.kv_off >= 0 else None, batch.positions,

@@ -300,16 +300,19 @@ def _group_rms(x: torch.Tensor, groups: int, eps: float) -> torch.Tensor:
 def stream_add_group_norm(x: torch.Tensor, y: Optional[torch.Tensor], y2: Optional[torch.Tensor],
                           bias: Optional[torch.Tensor], w1: torch.Tensor,
                           w2: Optional[torch.Tensor], groups: int, eps: float,
-                          out1: torch.Tensor, out2: Optional[torch.Tensor] = None) -> None:
+                          out1: torch.Tensor, out2: Optional[torch.Tensor] = None,
+                          shift: Optional[tuple] = None) -> None:
     """x += y + bias + y2 in place (fp32 stream; y [T, d] and bias [d] in the activation type,
     y2 [T, d] fp32; each may be None), then the RMS norm of the new x in `groups` equal
     consecutive parts (each divided by its own root mean square), written twice: out1 with the
     weights w1 and out2 with w2 (None: one output).  One pass over the row serves the residual
     update and both norms of a layer whose mixer and feed-forward read differently-weighted
-    norms of the same stream."""
+    norms of the same stream.  shift = (mu, state, seq_slot, positions): out1 additionally goes
+    through token_shift(single=True) inside the same kernel (batches whose every row is a
+    sequence of its own: decode steps)."""
     if _native(x):
         torch.ops.akap_stream.add_group_norm(out1, out2, x, y, y2, bias, w1, w2, int(groups),
-                                             float(eps))
+                                             float(eps), *(shift or (None, None, None, None)))
         return
     if y is not None:
         x.add_(y.float())
@@ -318,7 +321,12 @@ def stream_add_group_norm(x: torch.Tensor, y: Optional[torch.Tensor], y2: Option
     if y2 is not None:
         x.add_(y2)
     n = _group_rms(x, groups, eps)
-    out1.copy_((n * w1.float()).to(out1.dtype))
+    if shift is None:
+        out1.copy_((n * w1.float()).to(out1.dtype))
+    else:
+        mu, state, seq_slot, positions = shift
+        token_shift((n * w1.float()).to(out1.dtype), mu, state, seq_slot, positions, out1,
+                    single=True)
     if out2 is not None:
         out2.copy_((n * w2.float()).to(out2.dtype))
 

@@ -60,6 +60,41 @@ def test_add_group_norm_kernel(dtype, d, groups):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("d,groups", [(54, 9), (2048, 4), (6144, 1)])
+def test_add_group_norm_with_shift_kernel(dtype, d, groups):
+    """Decode steps: the token shift of the first output inside the norm kernel equals the norm
+    followed by token_shift(single=True), state included."""
+    g, dt = gen(d), DT[dtype]
+    T = 5
+    x = torch.randn(T, d, generator=g)
+    y = torch.randn(T, d, generator=g).to(dt)
+    w1, w2 = 1 + 0.3 * torch.randn(d, generator=g), 1 + 0.3 * torch.randn(d, generator=g)
+    mu = torch.rand(d, generator=g)
+    state = torch.randn(4, d, generator=g).to(dt)
+    slot = torch.tensor([2, 0, 3, 1, -1], dtype=torch.int32)
+    pos = torch.tensor([5, 0, 9, 4, 0])
+    res = []
+    for dev in ("cpu", "cuda"):
+        xx, st = x.clone().to(dev), state.clone().to(dev)
+        o1 = torch.zeros(T, d, dtype=dt, device=dev)
+        o2 = torch.zeros(T, d, dtype=dt, device=dev)
+        sops.stream_add_group_norm(xx, y.to(dev), None, None, w1.to(dev), w2.to(dev), groups, 1e-5,
+                                   o1, o2, shift=(mu.to(dev), st, slot.to(dev), pos.to(dev)))
+        res.append((xx, o1[:4], o2, st))
+    close(res[1][0], res[0][0], "float32")
+    for a, b in zip(res[1][1:], res[0][1:]):
+        close(a, b, dtype)
+    # against the two-step form on the GPU itself
+    xx, st = x.clone().cuda(), state.clone().cuda()
+    n1 = torch.zeros(T, d, dtype=dt, device="cuda")
+    h = torch.zeros(T, d, dtype=dt, device="cuda")
+    sops.stream_add_group_norm(xx, y.cuda(), None, None, w1.cuda(), None, groups, 1e-5, n1)
+    sops.token_shift(n1, mu.cuda(), st, slot.cuda(), pos.cuda(), h, single=True)
+    close(h[:4], res[1][1], dtype)      # (the compiler may contract the blend differently)
+    assert torch.equal(st, res[1][3])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("d", [70, 72, 2048])
 def test_token_shift_kernel(dtype, d):
     g, dt = gen(1), DT[dtype]
