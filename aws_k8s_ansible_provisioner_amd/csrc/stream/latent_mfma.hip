@@ -281,10 +281,31 @@ struct CoopSmem {
   static constexpr int DK = 32 * NV + 16 * NKR;
   static constexpr size_t q_bytes = (size_t)32 * q_pitch(DK) * sizeof(bf16);
   static constexpr size_t p_bytes = (size_t)4 * 2 * 64 * sizeof(bf16x8);
-  static constexpr size_t bytes = q_bytes + p_bytes + 2 * 4 * 32 * sizeof(float);
+  static constexpr size_t fixed = q_bytes + p_bytes + 2 * 4 * 32 * sizeof(float);
+  // + one cache row index per 32-key block of the workgroup's key range
+  static size_t bytes(const LatentAttnParams& p) {
+    return fixed + (size_t)p.max_blocks * (p.BS / 32) * sizeof(int32_t);
+  }
 };
 
+// The cache rows of the 32-key blocks [jb, je] of a sequence -> LDS, once: a block's row is
+// then an LDS read away instead of a block-table load ahead of every fragment load (with it,
+// a 128-key step was a chain of six dependent global loads, 17 us for a lone workgroup).
 template <int NV, int NKR>
+__device__ __forceinline__ void coop_load_rows(unsigned char* smem, const LatentAttnParams& p,
+                                               const int32_t* __restrict__ bt, int jb, int je) {
+  int32_t* sm_rows = reinterpret_cast<int32_t*>(smem + CoopSmem<NV, NKR>::fixed);
+  const int n = (je - jb) / 32 + 1;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const int j0 = jb + 32 * i;
+    const int bi = j0 / p.BS;
+    int blk = bi < p.max_blocks ? bt[bi] : 0;
+    if (blk < 0 || blk >= p.NB) blk = 0;
+    sm_rows[i] = blk * p.BS + (j0 - bi * p.BS);
+  }
+}
+
+template <int NV, int NKR, int KB>
 __device__ __forceinline__ void coop_attend(CoopState<NV / 4>& st, const LatentAttnParams& p,
                                             const int32_t* __restrict__ bt, unsigned char* smem,
                                             int pos, int pos_min, int jb, int je) {
@@ -300,29 +321,63 @@ __device__ __forceinline__ void coop_attend(CoopState<NV / 4>& st, const LatentA
   bf16x8* sm_p = reinterpret_cast<bf16x8*>(smem + SM::q_bytes);          // [4][2][64]
   float* sm_max = reinterpret_cast<float*>(smem + SM::q_bytes + SM::p_bytes);   // [4][32]
   float* sm_sum = sm_max + 4 * 32;                                              // [4][32]
-  auto row_of = [&](int j0) -> size_t {
-    const int bi = j0 / p.BS;
-    int blk = bi < p.max_blocks ? bt[bi] : 0;
-    if (blk < 0 || blk >= p.NB) blk = 0;
-    return (size_t)blk * p.BS + (j0 - bi * p.BS);
+  const int32_t* sm_rows = reinterpret_cast<const int32_t*>(smem + SM::fixed);  // coop_load_rows
+  auto row_of = [&](int j0) -> size_t { return (size_t)sm_rows[(j0 - jb) >> 5]; };
+  // Fragment loads are issued in batches AHEAD of the products that use them (a load issued
+  // right before its product makes a 128-key step a chain of 68 memory latencies: 17 us for a
+  // lone workgroup): K in double-buffered batches of KB k-steps, the latent fragments of a
+  // 32-key block one block ahead, the first block's before the softmax.  (Prefill: KB = 4 and
+  // two waves per SIMD; decode: KB = 12 and one.)
+  constexpr int NKB = (KS + KB - 1) / KB;
+  auto load_v = [&](bf16x8 (&vf)[2 * NVW], int jk) {
+    const bf16* vp = vg + (((row_of(jk) >> 3) + hf) * R + 32 * (wave * NVW) + col) * 8;
+#pragma unroll
+    for (int dt = 0; dt < NVW; ++dt) {
+      vf[2 * dt] = *reinterpret_cast<const bf16x8*>(vp + (size_t)(32 * dt) * 8);
+      vf[2 * dt + 1] = *reinterpret_cast<const bf16x8*>(vp + ((size_t)2 * R + 32 * dt) * 8);
+    }
   };
+  // the first K batch of a step is requested a step ahead (before the previous step's softmax)
+  bf16x8 ka[KB], kb2[KB];
+  auto load_k0 = [&](int jw) {
+    const bf16* kp = cache + (row_of(jw) + krow) * DK + 8 * hf;
+#pragma unroll
+    for (int c = 0; c < KB; ++c)
+      if (c < KS) ka[c] = *reinterpret_cast<const bf16x8*>(kp + 16 * c);
+  };
+  if (jb + 32 * wave <= je) load_k0(jb + 32 * wave);
   for (int j0 = jb; j0 <= je; j0 += 128) {
     const int jw = j0 + 32 * wave;
     const bool active = jw <= je;                    // (wave-uniform)
     float sv[16];
     float bmax = -INFINITY;
+    bf16x8 va[2 * NVW], vb[2 * NVW];
     if (active) {
       const bf16* kp = cache + (row_of(jw) + krow) * DK + 8 * hf;
       f32x16 s;
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
-      for (int c = 0; c < KS; ++c) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + 16 * c);
-        const bf16x8 qf = *reinterpret_cast<const bf16x8*>(qcol + 16 * c);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf, s, 0, 0, 0);
-        // at most 12 K fragments are requested ahead of the products that use them
-        if (c % 12 == 11) __builtin_amdgcn_sched_barrier(0);
+      for (int b = 0; b < NKB; ++b) {
+        // the next batch goes out before this batch's products
+        if (b + 1 < NKB) {
+#pragma unroll
+          for (int c = 0; c < KB; ++c)
+            if ((b + 1) * KB + c < KS) {
+              const bf16x8 f = *reinterpret_cast<const bf16x8*>(kp + 16 * ((b + 1) * KB + c));
+              if (b % 2 == 0) kb2[c] = f; else ka[c] = f;
+            }
+        } else {
+          load_v(va, j0);                            // block 0 of the step: always a valid block
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < KB; ++c)
+          if (b * KB + c < KS) {
+            const bf16x8 qf = *reinterpret_cast<const bf16x8*>(qcol + 16 * (b * KB + c));
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b % 2 == 0 ? ka[c] : kb2[c], qf, s, 0, 0, 0);
+          }
+        __builtin_amdgcn_sched_barrier(0);
       }
       if (jw + 31 <= pos_min) {
 #pragma unroll
@@ -339,7 +394,10 @@ __device__ __forceinline__ void coop_attend(CoopState<NV / 4>& st, const LatentA
         }
       }
       bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    } else {
+      load_v(va, j0);
     }
+    if (jw + 128 <= je) load_k0(jw + 128);           // (both K buffers are free here)
     if (hf == 0) sm_max[wave * 32 + col] = bmax;
     __syncthreads();
     const float bm = fmaxf(fmaxf(sm_max[col], sm_max[32 + col]),
@@ -375,16 +433,20 @@ __device__ __forceinline__ void coop_attend(CoopState<NV / 4>& st, const LatentA
     for (int kb = 0; kb < 4; ++kb) {
       const int jk = j0 + 32 * kb;
       if (jk <= je) {                                // (uniform over the workgroup)
+        if (kb + 1 < 4 && jk + 32 <= je) {           // the next block's fragments go out first
+          if (kb % 2 == 0) load_v(vb, jk + 32); else load_v(va, jk + 32);
+        }
         const bf16x8 p0 = sm_p[(kb * 2 + 0) * 64 + lane];
         const bf16x8 p1 = sm_p[(kb * 2 + 1) * 64 + lane];
-        const bf16* vp = vg + (((row_of(jk) >> 3) + hf) * R + 32 * (wave * NVW) + col) * 8;
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int dt = 0; dt < NVW; ++dt) {
-          const bf16x8 v0 = *reinterpret_cast<const bf16x8*>(vp + (size_t)(32 * dt) * 8);
-          const bf16x8 v1 = *reinterpret_cast<const bf16x8*>(vp + ((size_t)2 * R + 32 * dt) * 8);
-          st.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, p0, st.o[dt], 0, 0, 0);
-          st.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, st.o[dt], 0, 0, 0);
+          st.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kb % 2 == 0 ? va[2 * dt] : vb[2 * dt],
+                                                             p0, st.o[dt], 0, 0, 0);
+          st.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              kb % 2 == 0 ? va[2 * dt + 1] : vb[2 * dt + 1], p1, st.o[dt], 0, 0, 0);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   }
@@ -420,7 +482,7 @@ __device__ __forceinline__ void coop_init(CoopState<NVW>& st) {
 
 // Prefill: flat grid over (32-token sub-tile, head) units, one workgroup of 4 waves each
 template <int NV, int NKR>
-__global__ __launch_bounds__(256) void latent_prefill_coop_kernel(LatentAttnParams p) {
+__global__ __launch_bounds__(256, 2) void latent_prefill_coop_kernel(LatentAttnParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   constexpr int R = 32 * NV, NVW = NV / 4;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -440,6 +502,8 @@ __global__ __launch_bounds__(256) void latent_prefill_coop_kernel(LatentAttnPara
   const int rend = min(p.tile_row[tile] + p.tile_rows, qlen);
   const int r0 = p.tile_row[tile] + 32 * si;
   if (r0 >= rend || kv < qlen) return;
+  const int pos_last = kv - qlen + min(r0 + 31, rend - 1);
+  coop_load_rows<NV, NKR>(smem, p, p.block_tables + (size_t)b * p.max_blocks, 0, pos_last);
   coop_load_queries<NV, NKR>(smem, p, [&](int c, int& t, int& hh) {
     t = qs0 + (r0 + c < rend ? r0 + c : r0);
     hh = h;
@@ -450,8 +514,7 @@ __global__ __launch_bounds__(256) void latent_prefill_coop_kernel(LatentAttnPara
   CoopState<NVW> st;
   coop_init(st);
   const int pos_first = kv - qlen + r0;
-  const int pos_last = kv - qlen + min(r0 + 31, rend - 1);
-  coop_attend<NV, NKR>(st, p, p.block_tables + (size_t)b * p.max_blocks, smem, kv - qlen + r,
+  coop_attend<NV, NKR, 4>(st, p, p.block_tables + (size_t)b * p.max_blocks, smem, kv - qlen + r,
                        pos_first, 0, pos_last);
   if (!valid) return;
   const float f = st.l > 0.f ? 1.0f / st.l : 0.f;
@@ -488,11 +551,13 @@ __global__ __launch_bounds__(256) void latent_decode_coop_kernel(LatentAttnParam
   CoopState<NVW> st;
   coop_init(st);
   if (jb <= je) {                                    // (workgroup-uniform)
+    coop_load_rows<NV, NKR>(smem, p, p.block_tables + (size_t)b * p.max_blocks, jb, je);
     coop_load_queries<NV, NKR>(smem, p, [&](int c, int& t, int& hh) {
       t = b;
       hh = c0 + c < p.H ? c0 + c : c0;
     });
-    coop_attend<NV, NKR>(st, p, p.block_tables + (size_t)b * p.max_blocks, smem, pos1, pos1, jb, je);
+    coop_attend<NV, NKR, 12>(st, p, p.block_tables + (size_t)b * p.max_blocks, smem, pos1, pos1, jb,
+                            je);
   }
   if (!valid) return;
   if (p.num_parts == 1) {
@@ -550,7 +615,7 @@ void launch_prefill(const LatentAttnParams& p, hipStream_t s) {
   if constexpr (NV >= 8) {
     const int units = p.num_tiles * (p.tile_rows / 32);
     const unsigned grid = (unsigned)((units + 7) / 8 * 8) * p.H;
-    latent_prefill_coop_kernel<NV, NKR><<<grid, 256, CoopSmem<NV, NKR>::bytes, s>>>(p);
+    latent_prefill_coop_kernel<NV, NKR><<<grid, 256, CoopSmem<NV, NKR>::bytes(p), s>>>(p);
     return;
   }
   constexpr size_t per_wave = (size_t)32 * q_pitch(DK) * sizeof(bf16);
@@ -573,7 +638,7 @@ void launch_decode(const LatentAttnParams& p, hipStream_t s) {
   constexpr int DK = 32 * NV + 16 * NKR;
   const dim3 grid(p.B, (p.H + 31) / 32, p.num_parts);
   if constexpr (NV >= 8)
-    latent_decode_coop_kernel<NV, NKR><<<grid, 256, CoopSmem<NV, NKR>::bytes, s>>>(p);
+    latent_decode_coop_kernel<NV, NKR><<<grid, 256, CoopSmem<NV, NKR>::bytes(p), s>>>(p);
   else
     latent_decode_mfma_kernel<NV, NKR><<<grid, 64, (size_t)32 * q_pitch(DK) * sizeof(bf16), s>>>(p);
   if (p.num_parts > 1)

@@ -500,6 +500,8 @@ akap_stream::LatentAttnParams latent_mfma_params(const Tensor& out, const Tensor
                   block_tables.stride(1) == 1 && seq_lens.scalar_type() == at::kInt &&
                   block_tables.size(0) >= seq_lens.numel(), "block_tables / seq_lens");
   TORCH_CHECK(cache.size(0) * BS < (1LL << 31), "cache has too many rows");
+  // (wide latents keep one row index per 32-key block of a sequence in LDS)
+  TORCH_CHECK(block_tables.size(1) * (BS / 32) <= 16384, "block table too long for the LDS");
   akap_stream::LatentAttnParams p{};
   p.out = out.data_ptr();
   p.q_lat = q_lat.data_ptr();

@@ -458,7 +458,7 @@ def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q: torch.Tensor, ro
 
 
 def latent_mfma_ok(cache: torch.Tensor, vgroups: Optional[torch.Tensor], kv_rank: int,
-                   q: torch.Tensor, rot_off: int, scale: float) -> bool:
+                   q: torch.Tensor, rot_off: int, scale: float, max_blocks: int = 0) -> bool:
     """The matrix-core kernels take a bf16 GPU cache with its grouped copy, latent / rotated
     sizes they were built for, 32-token-aligned blocks and 16-byte-aligned query rows."""
     if vgroups is None or not cache.is_cuda or cache.dtype != torch.bfloat16:
@@ -466,7 +466,7 @@ def latent_mfma_ok(cache: torch.Tensor, vgroups: Optional[torch.Tensor], kv_rank
     load_native(required=True)
     return (torch.ops.akap_stream.latent_mfma_supported(kv_rank, cache.shape[2] - kv_rank)
             and cache.shape[1] % 32 == 0 and rot_off % 8 == 0 and q.shape[2] % 8 == 0
-            and scale > 0)
+            and scale > 0 and max_blocks * (cache.shape[1] // 32) <= 16384)
 
 
 def latent_attention_prefill(out: torch.Tensor, q_lat: torch.Tensor, q: torch.Tensor,
@@ -478,7 +478,7 @@ def latent_attention_prefill(out: torch.Tensor, q_lat: torch.Tensor, q: torch.Te
     before q_start[first_seq] belong to single-token sequences and are left alone): on the
     matrix cores when latent_mfma_ok, driven by the scheduler's tile map (tile_seq / tile_row:
     sequence and first chunk row of a tile of tile_rows tokens), else the row kernel."""
-    if latent_mfma_ok(cache, vgroups, q_lat.shape[2], q, rot_off, scale):
+    if latent_mfma_ok(cache, vgroups, q_lat.shape[2], q, rot_off, scale, block_tables.shape[1]):
         torch.ops.akap_stream.latent_attention_prefill_mfma(
             out, q_lat, q, rot_off, cache, vgroups, block_tables, seq_lens, q_start, tile_seq,
             tile_row, tile_rows, float(scale))
@@ -506,7 +506,7 @@ def latent_attention_decode(out: torch.Tensor, q_lat: torch.Tensor, q: torch.Ten
     row, left unwritten).  On the matrix cores (latent_mfma_ok) the heads of a token are the
     columns of one tile and the keys are cut into num_parts partitions of whole 32-key blocks,
     one wave each, merged by a second launch (workspace from latent_decode_workspace)."""
-    if latent_mfma_ok(cache, vgroups, q_lat.shape[2], q, rot_off, scale):
+    if latent_mfma_ok(cache, vgroups, q_lat.shape[2], q, rot_off, scale, block_tables.shape[1]):
         ws_ml, ws_o = workspace if (workspace is not None and num_parts > 1) else (None, None)
         torch.ops.akap_stream.latent_attention_decode_mfma(
             out, q_lat, q, rot_off, cache, vgroups, block_tables, seq_lens, float(scale), ws_ml,
