@@ -11,13 +11,14 @@
 // one exchange between the lane halves.  The K rows are loaded in the order (bits 2 and 3 of
 // the row swapped) that makes a lane's S^T accumulators exactly the 8 keys of one group, so P
 // moves from accumulator to operand without lane traffic and the C^T operand is one 16-byte
-// load from the grouped copy.  The query tile (32 columns x (R + r)) lives in LDS: at R = 512
-// the output accumulators alone are 256 registers.  K and C fragments come straight from
-// global memory (L1 / L2: the heads of a token tile are workgroups of one XCD).
+// load from the grouped copy.  The query tile (32 columns x (R + r)) lives in LDS.  K and C
+// fragments come straight from global memory (L1 / L2: the heads of a token tile are
+// workgroups of one XCD).
 //
-// Prefill: a wave owns 32 consecutive tokens of one head (causal mask only in the blocks that
-// cross its positions).  Decode: the 32 columns are the heads of one token; the key range is
-// cut into partitions merged by a second launch.
+// Prefill: the 32 columns are consecutive tokens of one head (causal mask only in the blocks
+// that cross its positions).  Decode: the 32 columns are the heads of one token; the key range
+// is cut into partitions merged by a second launch.  Narrow latents (R <= 128): one wave per
+// tile.  Wide latents: four waves per tile (see below).
 #include "../kernels/common.h"
 #include "stream.h"
 
@@ -612,24 +613,15 @@ __global__ __launch_bounds__(128) void latent_decode_merge_kernel(LatentAttnPara
 template <int NV, int NKR>
 void launch_prefill(const LatentAttnParams& p, hipStream_t s) {
   constexpr int DK = 32 * NV + 16 * NKR;
-  if constexpr (NV >= 8) {
-    const int units = p.num_tiles * (p.tile_rows / 32);
-    const unsigned grid = (unsigned)((units + 7) / 8 * 8) * p.H;
-    latent_prefill_coop_kernel<NV, NKR><<<grid, 256, CoopSmem<NV, NKR>::bytes(p), s>>>(p);
-    return;
-  }
-  constexpr size_t per_wave = (size_t)32 * q_pitch(DK) * sizeof(bf16);
   const int units = p.num_tiles * (p.tile_rows / 32);
-  // as many heads per workgroup as fit 64 KB of LDS
-  if (4 * per_wave <= 64 * 1024) {
-    const unsigned grid = (unsigned)((units + 7) / 8 * 8) * ((p.H + 3) / 4);
-    latent_prefill_mfma_kernel<NV, NKR, 4><<<grid, 256, 4 * per_wave, s>>>(p);
-  } else if (2 * per_wave <= 64 * 1024) {
-    const unsigned grid = (unsigned)((units + 7) / 8 * 8) * ((p.H + 1) / 2);
-    latent_prefill_mfma_kernel<NV, NKR, 2><<<grid, 128, 2 * per_wave, s>>>(p);
+  const unsigned padded = (unsigned)((units + 7) / 8 * 8);
+  if constexpr (NV >= 8) {
+    latent_prefill_coop_kernel<NV, NKR><<<padded * p.H, 256, CoopSmem<NV, NKR>::bytes(p), s>>>(p);
   } else {
-    const unsigned grid = (unsigned)((units + 7) / 8 * 8) * p.H;
-    latent_prefill_mfma_kernel<NV, NKR, 1><<<grid, 64, per_wave, s>>>(p);
+    // narrow latents: one wave per tile and head, 4 heads per workgroup
+    constexpr size_t per_wave = (size_t)32 * q_pitch(DK) * sizeof(bf16);
+    static_assert(4 * per_wave <= 64 * 1024, "query tiles of four heads fit the LDS");
+    latent_prefill_mfma_kernel<NV, NKR, 4><<<padded * ((p.H + 3) / 4), 256, 4 * per_wave, s>>>(p);
   }
 }
 
