@@ -637,7 +637,54 @@ void launch_decode(const LatentAttnParams& p, hipStream_t s) {
     latent_decode_merge_kernel<<<dim3(p.B, p.H), 128, p.num_parts * sizeof(float), s>>>(p);
 }
 
+// ---- per-head products of small batches ------------------------------------------------------
+// out[h, t, n] = sum_k a[h, t, k] w[h, n, k] for a few rows t (decode steps): one wave per
+// 32 x 32 tile of one head, both operands contiguous in k (16-byte fragment loads), k in
+// batches of 8 MFMA steps whose loads go out together.  The library's batched GEMM takes
+// 12-14 us for these 0.1 GFLOP products at 64 rows.
+__global__ __launch_bounds__(64) void head_matmul_kernel(bf16* __restrict__ out,
+                                                         const bf16* __restrict__ a, int64_t a_hs,
+                                                         int64_t a_ts, const bf16* __restrict__ w,
+                                                         int T, int N, int K) {
+  const int lane = threadIdx.x;
+  const int col = lane & 31, hf = lane >> 5;
+  const int ntn = N / 32;
+  const int h = blockIdx.y, nt = blockIdx.x % ntn, mt = blockIdx.x / ntn;
+  const int row = min(mt * 32 + col, T - 1);
+  const bf16* ap = a + (size_t)h * a_hs + (size_t)row * a_ts + 8 * hf;
+  const bf16* wp = w + ((size_t)h * N + nt * 32 + col) * K + 8 * hf;
+  f32x16 acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 128) {
+    bf16x8 af[8], wf[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+      if (k0 + 16 * c < K) {                         // (uniform)
+        af[c] = *reinterpret_cast<const bf16x8*>(ap + k0 + 16 * c);
+        wf[c] = *reinterpret_cast<const bf16x8*>(wp + k0 + 16 * c);
+      }
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+      if (k0 + 16 * c < K) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[c], wf[c], acc, 0, 0, 0);
+  }
+  // accumulator register i: row 8 (i >> 2) + 4 hf + (i & 3) of the tile, column col
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int r = mt * 32 + 8 * (i >> 2) + 4 * hf + (i & 3);
+    if (r < T) out[((size_t)h * T + r) * N + nt * 32 + col] = (bf16)acc[i];
+  }
+}
+
 }  // namespace
+
+void launch_head_matmul(void* out, const void* a, int64_t a_hs, int64_t a_ts, const void* w, int H,
+                        int T, int N, int K, hipStream_t s) {
+  if (H <= 0 || T <= 0) return;
+  const dim3 grid((N / 32) * ((T + 31) / 32), H);
+  head_matmul_kernel<<<grid, 64, 0, s>>>((bf16*)out, (const bf16*)a, a_hs, a_ts, (const bf16*)w, T,
+                                         N, K);
+}
 
 // the latent / rotated sizes the matrix kernels are built for
 bool latent_mfma_sizes(int R, int r) {

@@ -142,6 +142,10 @@ bool latent_mfma_sizes(int R, int r);
 void launch_latent_prefill_mfma(const LatentAttnParams& p, hipStream_t s);
 void launch_latent_decode_mfma(const LatentAttnParams& p, hipStream_t s);
 
+// out [H, T, N] = a [H, T, K] (strides a_hs / a_ts, unit in k) x w [H, N, K]^T, bf16, K % 16 == 0,
+// N % 32 == 0, 16-byte aligned rows; meant for a few rows (one wave per 32 x 32 tile)
+void launch_head_matmul(void* out, const void* a, int64_t a_hs, int64_t a_ts, const void* w, int H,
+                        int T, int N, int K, hipStream_t s);
 void launch_head_gate(void* out, int out_stride, const void* o, const void* gate, int gate_stride,
                       bool per_head, int rows, int H, int V, bool f32, hipStream_t s);
 void launch_xielu(void* out, int out_stride, const void* x, int x_stride, const void* bias,

@@ -566,6 +566,23 @@ bool latent_mfma_supported(int64_t R, int64_t r) {
   return akap_stream::latent_mfma_sizes((int)R, (int)r);
 }
 
+void head_matmul(Tensor out, Tensor a, Tensor w) {
+  CHECK_GPU(out); CHECK_GPU(a); CHECK_GPU(w); CHECK_CONTIG(out); CHECK_CONTIG(w);
+  TORCH_CHECK(a.dim() == 3 && w.dim() == 3 && out.dim() == 3 && a.stride(2) == 1, "head_matmul: ranks");
+  const int64_t H = a.size(0), T = a.size(1), K = a.size(2), N = w.size(1);
+  TORCH_CHECK(w.size(0) == H && w.size(2) == K && out.size(0) == H && out.size(1) == T &&
+                  out.size(2) == N, "head_matmul: shapes");
+  for (const Tensor* t : {&out, &a, &w})
+    TORCH_CHECK(t->scalar_type() == at::kBFloat16, "head_matmul is bf16");
+  TORCH_CHECK(K % 16 == 0 && N % 32 == 0 && a.stride(0) % 8 == 0 && a.stride(1) % 8 == 0 &&
+                  (uintptr_t)a.data_ptr() % 16 == 0 && (uintptr_t)w.data_ptr() % 16 == 0,
+              "head_matmul: sizes / alignment");
+  TORCH_CHECK(H <= 65535 && (N / 32) * ((T + 31) / 32) < (1LL << 31), "head_matmul: grid");
+  const c10::DeviceGuard g(a.device());
+  akap_stream::launch_head_matmul(out.data_ptr(), a.data_ptr(), a.stride(0), a.stride(1),
+                                  w.data_ptr(), (int)H, (int)T, (int)N, (int)K, cur_stream());
+}
+
 void head_gate(Tensor out, Tensor o, Tensor gate) {
   CHECK_GPU(out); CHECK_GPU(o); CHECK_GPU(gate); CHECK_CONTIG(o); CHECK_LAST_CONTIG(out);
   CHECK_LAST_CONTIG(gate);
@@ -705,6 +722,7 @@ TORCH_LIBRARY(akap_stream, m) {
   m.def("latent_attention(Tensor(a!) out, Tensor q_lat, Tensor q, int rot_off, Tensor cache, "
         "Tensor block_tables, Tensor seq_lens, Tensor? q_start, Tensor positions, float scale) "
         "-> ()");
+  m.def("head_matmul(Tensor(a!) out, Tensor a, Tensor w) -> ()");
   m.def("head_gate(Tensor(a!) out, Tensor o, Tensor gate) -> ()");
   m.def("xielu(Tensor(a!) out, Tensor x, Tensor? bias, Tensor act) -> ()");
   m.def("moe_route(Tensor(a!) ids, Tensor(b!) w, Tensor h, Tensor router, Tensor? correction, "
@@ -722,6 +740,7 @@ TORCH_LIBRARY_IMPL(akap_stream, CUDA, m) {
   m.impl("latent_attention", &latent_attention);
   m.impl("latent_attention_prefill_mfma", &latent_attention_prefill_mfma);
   m.impl("latent_attention_decode_mfma", &latent_attention_decode_mfma);
+  m.impl("head_matmul", &head_matmul);
   m.impl("head_gate", &head_gate);
   m.impl("xielu", &xielu);
   m.impl("moe_route", &moe_route);

@@ -55,8 +55,8 @@ class LatentLayerWeights:
     dq_norm: torch.Tensor               # fp32 [q_rank]
     dkv_norm: Optional[torch.Tensor]    # fp32 [kv_rank]
     w_uq: torch.Tensor                  # [H (D + r), q_rank]
-    w_uk: torch.Tensor                  # [H, D, R]: q_lat = q_unrot @ w_uk
-    w_uv: torch.Tensor                  # [H, R, V]: o = o_lat @ w_uv
+    w_uk: torch.Tensor                  # [H, R, D]: q_lat[h] = q_unrot[h] @ w_uk[h]^T
+    w_uv: torch.Tensor                  # [H, V, R]: o[h] = o_lat[h] @ w_uv[h]^T
     w_out: torch.Tensor                 # [d, H V (+ ff)] = [W_o | W_down]
     b_out: Optional[torch.Tensor]       # [d]
     cos_sin: torch.Tensor
@@ -150,8 +150,8 @@ class PuputarLM:
                 dq_norm=rand(m.q_rank, s=0.1, mean=1.0, dt=f32),
                 dkv_norm=rand(m.kv_rank, s=0.1, mean=1.0, dt=f32) if own else None,
                 w_uq=rand(m.heads * (m.dim + m.rot_dim), m.q_rank, s=sq),
-                w_uk=rand(m.heads, m.dim, m.kv_rank, s=sr),
-                w_uv=rand(m.heads, m.kv_rank, m.vdim, s=sr),
+                w_uk=rand(m.heads, m.kv_rank, m.dim, s=sr),
+                w_uv=rand(m.heads, m.vdim, m.kv_rank, s=sr),
                 w_out=rand(d, hv), b_out=None, cos_sin=self._table(m.rot), hv=hv)
             ml = ls.mlp
             if ml is not None:
@@ -180,10 +180,11 @@ class PuputarLM:
         out = [(p + "norm1", lw.norm1, same), (p + "shift", lw.shift, same),
                (p + "mix.dq", lw.w_in[:m.q_rank], same), (p + "mix.dq.norm", lw.dq_norm, same),
                (p + "mix.uq", lw.w_uq, same),
-               # [H D, R] -> [H, D, R] and [H V, R] -> [H, R, V]
-               (p + "mix.uk", lw.w_uk, lambda t: self._want(t, (H * D, R)).reshape(H, D, R)),
-               (p + "mix.uv", lw.w_uv,
-                lambda t: self._want(t, (H * V, R)).reshape(H, V, R).transpose(1, 2)),
+               # [H D, R] -> [H, R, D] and [H V, R] -> [H, V, R]: both contiguous in the index
+               # their product contracts over
+               (p + "mix.uk", lw.w_uk,
+                lambda t: self._want(t, (H * D, R)).reshape(H, D, R).transpose(1, 2)),
+               (p + "mix.uv", lw.w_uv, lambda t: self._want(t, (H * V, R)).reshape(H, V, R)),
                (p + "mix.g", lw.w_in[lw.g_off:lw.g_off + m.gate_rows], same),
                (p + "mix.o", lw.w_out[:, :lw.hv], same)]
         if lw.kv_off >= 0:
@@ -225,8 +226,8 @@ class PuputarLM:
         sd = {}
         for i, lw in enumerate(self.layers):
             m = lw.spec.mixer
-            sd[f"l{i}.mix.uk"] = lw.w_uk.reshape(m.heads * m.dim, m.kv_rank).clone()
-            sd[f"l{i}.mix.uv"] = lw.w_uv.transpose(1, 2).reshape(m.heads * m.vdim, m.kv_rank).clone()
+            sd[f"l{i}.mix.uk"] = lw.w_uk.transpose(1, 2).reshape(m.heads * m.dim, m.kv_rank).clone()
+            sd[f"l{i}.mix.uv"] = lw.w_uv.reshape(m.heads * m.vdim, m.kv_rank).clone()
         for name, t, _ in self._all_names():
             if name not in sd:
                 sd[name] = t.clone()
@@ -442,10 +443,10 @@ class PuputarLM:
                              0, lw.kv_off, eps, v_caches[r] if lw.kv_off >= 0 else None)
             q = self._linear(cq, lw.w_uq).view(T, H, D + rd)
             sops.rotate_heads_(q, batch.positions, lw.cos_sin, D)
-            q_lat = torch.bmm(q[:, :, :D].transpose(0, 1), lw.w_uk)           # [H, T, R]
+            q_lat = sops.head_matmul(q[:, :, :D].transpose(0, 1), lw.w_uk)    # [H, T, R]
             o_lat = torch.empty(H, T, R, dtype=dt, device=dev)
             self._attention(m, o_lat, q_lat, q, batch, k_caches[r], v_caches[r])
-            o = torch.bmm(o_lat, lw.w_uv)                                      # [H, T, V]
+            o = sops.head_matmul(o_lat, lw.w_uv)                               # [H, T, V]
             cat = torch.empty(T, lw.hv + lw.ff, dtype=dt, device=dev)
             sops.head_gate(o, proj[:, lw.g_off:lw.g_off + m.gate_rows], cat[:, :lw.hv])
             ml = lw.spec.mlp

@@ -515,6 +515,26 @@ def latent_attention_decode(out: torch.Tensor, q_lat: torch.Tensor, q: torch.Ten
     latent_attention(out, q_lat, q, rot_off, cache, block_tables, seq_lens, None, positions, scale)
 
 
+# rows up to which the per-head products take the one-wave-per-tile kernel
+HEAD_MATMUL_ROWS = 256
+
+
+def head_matmul(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """out[h] = a[h] @ w[h]^T for every head: a [H, T, K] (any head / row strides, unit stride in
+    k: a view of [T, H, n] rows is fine), w [H, N, K].  A few rows of bf16 on the GPU (decode
+    steps) run a small matrix-core kernel; everything else the library's batched GEMM."""
+    H, T, K = a.shape
+    N = w.shape[1]
+    if (a.is_cuda and a.dtype == torch.bfloat16 and 0 < T <= HEAD_MATMUL_ROWS and K % 16 == 0
+            and N % 32 == 0 and a.stride(2) == 1 and a.stride(0) % 8 == 0 and a.stride(1) % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.is_contiguous()):
+        load_native(required=True)
+        out = torch.empty(H, T, N, dtype=a.dtype, device=a.device)
+        torch.ops.akap_stream.head_matmul(out, a, w)
+        return out
+    return torch.bmm(a, w.transpose(1, 2))
+
+
 def head_gate(o: torch.Tensor, gate: torch.Tensor, out: torch.Tensor) -> None:
     """out[t, h V + j] = o[h, t, j] * sigmoid(g), g = gate[t, h] when gate has H columns (one
     gate per head) or gate[t, h V + j] when it has H V (one per output entry).  o [H, T, V]

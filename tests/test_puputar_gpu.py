@@ -435,3 +435,18 @@ def test_engine_on_the_matrix_core_path(tmp_path, eager):
             check(replay(eng, reqs, sched), want, dtype)
         one = {"a": reqs["a"]}
         check(replay(eng, one, [[("a", 330)]] + [[("a", 1)]] * 60), want, dtype)
+
+
+@pytest.mark.parametrize("H,T,K,N", [(16, 64, 128, 512), (16, 64, 512, 128), (3, 1, 32, 96),
+                                     (5, 37, 48, 64), (6, 200, 96, 32), (2, 300, 64, 64), (4, 9, 20, 64)])
+def test_head_matmul_kernel(H, T, K, N):
+    """The per-head products of small batches (strided rows of a [T, H, n] buffer as well as
+    head-major rows) against the batched library GEMM in fp32; more rows than the kernel takes
+    and sizes off its grid go to the library."""
+    g = gen(H * T)
+    wide = (torch.randn(T, H, K + 16, generator=g) * 0.5).to(torch.bfloat16).cuda()
+    w = (torch.randn(H, N, K, generator=g) * K ** -0.5).to(torch.bfloat16).cuda()
+    a = wide[:, :, :K].transpose(0, 1)
+    want = torch.bmm(a.float(), w.float().transpose(1, 2))
+    close(sops.head_matmul(a, w), want, "bfloat16")
+    close(sops.head_matmul(a.contiguous(), w), want, "bfloat16")
