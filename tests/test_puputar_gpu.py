@@ -357,8 +357,8 @@ def _tile_map(q_start, seq_lens, first_seq, tile_rows):
             torch.tensor([t[2] for t in tiles], dtype=torch.int32))
 
 
-@pytest.mark.parametrize("H,D,r,R", [(3, 8, 16, 64), (6, 32, 16, 96), (4, 16, 32, 128),
-                                     (33, 8, 32, 256), (16, 128, 64, 512)])
+@pytest.mark.parametrize("H,D,r,R", [(3, 8, 16, 64), (6, 32, 16, 96), (4, 16, 32, 128), (2, 24, 16, 128),
+                                     (33, 8, 32, 256), (5, 16, 64, 256), (16, 128, 64, 512)])
 def test_latent_attention_matrix_core_kernels(H, D, r, R):
     """Prefill tiles (a chunk that continues a cached prefix, a whole prompt, a short one) and
     split decode on the matrix cores against the PyTorch op; one far key per sequence is made
