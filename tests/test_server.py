@@ -223,3 +223,38 @@ def test_bidetar_served_with_prefix_cache_and_sampling():
     hits = sum(float(ln.rsplit(" ", 1)[1]) for ln in text.splitlines()
                if ln.startswith("vllm:prefix_cache_hits_total"))
     assert hits >= 96  # the second request reused 3 full pages of the first
+
+
+def test_puputar_served_with_sampling_and_no_prefix_cache():
+    """The latent-attention design with per-sequence shift state behind the same OpenAI
+    endpoints: greedy completions are reproducible although the repeated prompt may NOT reuse
+    cached pages (a cached prefix does not hold the shift state at its end, so the engine
+    turns prefix caching off for this model), concurrent prompts share the slot pool, sampled
+    requests run too."""
+    from aws_k8s_ansible_provisioner_amd.engine.config import EngineConfig
+    from aws_k8s_ansible_provisioner_amd.server.api_server import build_app
+
+    app, ae = build_app(EngineConfig(model="tiny-puputar", served_model_name="p", device="cpu",
+                                     dtype="float32", max_model_len=256, max_num_seqs=2,
+                                     max_num_batched_tokens=48, block_size=32,
+                                     num_gpu_blocks=64, enable_prefix_caching=True))
+    prompt = list(range(10, 110))
+    with TestClient(app) as c:
+        outs = []
+        for _ in range(2):
+            r = c.post("/v1/completions", json={"prompt": prompt, "max_tokens": 6,
+                                                "temperature": 0.0})
+            assert r.status_code == 200, r.text
+            outs.append(r.json()["choices"][0]["text"])
+        assert outs[0] == outs[1]
+        # more prompts than sequence slots in one request: slots are handed on
+        r = c.post("/v1/completions", json={"prompt": [prompt[:20], prompt[:33], prompt[:7]],
+                                            "max_tokens": 4, "temperature": 0.0})
+        assert r.status_code == 200 and len(r.json()["choices"]) == 3
+        r = c.post("/v1/completions", json={"prompt": prompt[:50], "max_tokens": 5,
+                                            "temperature": 0.8, "top_p": 0.9, "seed": 3})
+        assert r.status_code == 200 and r.json()["usage"]["completion_tokens"] == 5
+        text = c.get("/metrics").text
+    hits = sum(float(ln.rsplit(" ", 1)[1]) for ln in text.splitlines()
+               if ln.startswith("vllm:prefix_cache_hits_total"))
+    assert hits == 0
