@@ -106,6 +106,7 @@ class PuputarLM:
         self._tables: dict = {}
         self.state: Optional[torch.Tensor] = None
         self._ws: Optional[tuple] = None
+        self._ws_kept: list = []
         self._seg_map: dict = {}
         self._init_weights(seed)
 
@@ -337,12 +338,19 @@ class PuputarLM:
         return min(max_parts, 64, max(1, math.ceil(256 / groups)))
 
     def _workspace(self, rows: int, heads: int, kv_rank: int, parts: int):
-        need = rows * heads * parts * kv_rank
-        if self._ws is None or self._ws[0] < need:
-            # grown on eager steps only: the runner warms every bucket before capturing it
-            self._ws = (need, sops.latent_decode_workspace(rows, heads, kv_rank, parts,
-                                                           self.device))
-        return self._ws[1]
+        """Partial softmax state of the split decode: (max, sum) per (row, head, partition) and
+        the unnormalised latent output.  Layers differ in heads and latent size, so both
+        buffers are checked; a buffer that has to grow (eager steps only: the runner warms a
+        bucket before capturing it) is kept alive, since captured graphs may still point at
+        it."""
+        n_ml, n_o = 2 * rows * heads * parts, rows * heads * parts * kv_rank
+        if self._ws is None or self._ws[0].numel() < n_ml or self._ws[1].numel() < n_o:
+            if self._ws is not None:
+                self._ws_kept.append(self._ws)
+                n_ml, n_o = max(n_ml, self._ws[0].numel()), max(n_o, self._ws[1].numel())
+            self._ws = (torch.empty(n_ml, dtype=torch.float32, device=self.device),
+                        torch.empty(n_o, dtype=torch.float32, device=self.device))
+        return self._ws
 
     def _attention(self, m: LatentAttentionSpec, o_lat, q_lat, q, batch: AttnBatch, cache,
                    groups) -> None:

@@ -450,3 +450,19 @@ def test_head_matmul_kernel(H, T, K, N):
     want = torch.bmm(a.float(), w.float().transpose(1, 2))
     close(sops.head_matmul(a, w), want, "bfloat16")
     close(sops.head_matmul(a.contiguous(), w), want, "bfloat16")
+
+
+def test_decode_workspace_serves_layers_of_unequal_heads_and_latents(tmp_path):
+    """A layer with few heads and a wide latent followed by one with many heads and a narrow
+    latent: the split-decode scratch has to fit both the per-(row, head) statistics and the
+    latent outputs of every layer, also in the captured graphs."""
+    cfg = oracle.make_config(width=64, vocab=41, groups=2, layers=[
+        oracle.make_layer(heads=4, dim=8, rot_dim=32, vdim=8, kv_rank=256, q_rank=24),
+        oracle.make_layer(heads=12, dim=16, rot_dim=16, vdim=4, kv_rank=64, q_rank=24, ff=32)])
+    W = oracle.random_weights(cfg, seed=4)
+    reqs = {"a": tokens(300, 41, 1), "b": tokens(200, 41, 2)}
+    want = {n: oracle.forward(cfg, W, t) for n, t in reqs.items()}
+    eng = engine(write_model(tmp_path, cfg, W), dtype="bfloat16", max_tokens=640, device="cuda")
+    assert eng.runner.graphs and all(g is not None for g in eng.runner.v_caches)
+    sched = [[("a", 280), ("b", 190)]] + [[("a", 1), ("b", 1)]] * 10 + [[("a", 10)]]
+    check(replay(eng, reqs, sched), want, "bfloat16")
